@@ -60,7 +60,7 @@ def plan_groups(needs: list, cache_of: list[int | None]) -> tuple[list[CacheGrou
         places = []
         for j, need in enumerate(mine):
             owner_need = theirs[j]
-            if (owner_need.num_kv_heads, owner_need.head_dim) != (need.num_kv_heads, need.head_dim):
+            if (owner_need.num_kv_heads, owner_need.head_dim, owner_need.value_size) != (need.num_kv_heads, need.head_dim, need.value_size):
                 raise ValueError(f"run entry {i} cannot read the cache of entry {owner}: head layout differs")
             if owner_need.window and (not need.window or need.window > owner_need.window):
                 raise ValueError(f"run entry {i} reads further back than entry {owner} keeps keys")

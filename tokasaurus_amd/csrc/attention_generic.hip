@@ -11,6 +11,9 @@
 //   K pages: [page][kv head][d / 8][P][8]   V pages: [page][kv head][P / 4][d][4]
 //   (key_offset and value_offset of common.h); block_table[req][pos / P] is the page of a position.
 // A query at position p sees positions max(0, p - window + 1) .. p (window <= 0: all).
+// Keys have d elements a head and values dv (dv = d in most models).  `sink` (null, or one
+// 32-bit number a query head): exp(sink) is added once to the softmax's denominator; it has no
+// key and no value.
 #include "common.h"
 
 #define AG_THREADS 256
@@ -21,7 +24,8 @@ __global__ __launch_bounds__(AG_THREADS) void paged_attention_generic_kernel(
     const T* __restrict__ q, int q_stride, T* __restrict__ out, int out_stride,
     const T* __restrict__ kcache, const T* __restrict__ vcache,
     const int* __restrict__ block_table, int table_stride, const int* __restrict__ token_req,
-    const int* __restrict__ positions, int nq, int nkv, int d, int P, int window, float scale) {
+    const int* __restrict__ positions, int nq, int nkv, int d, int dv, int P, int window, float scale,
+    const float* __restrict__ sink) {
   extern __shared__ float smem[];
   const int t = blockIdx.x, g = blockIdx.y;
   const int group = nq / nkv;
@@ -33,14 +37,14 @@ __global__ __launch_bounds__(AG_THREADS) void paged_attention_generic_kernel(
 
   float* qs = smem;                    // [group][d]
   float* Ks = qs + group * d;          // [CH][d + 1]
-  float* Vs = Ks + CH * (d + 1);       // [CH][d]
-  float* Ss = Vs + CH * d;             // [group][CH]
+  float* Vs = Ks + CH * (d + 1);       // [CH][dv]
+  float* Ss = Vs + CH * dv;            // [group][CH]
   float* st_m = Ss + group * CH;       // [group] running maximum
   float* st_l = st_m + group;          // [group] running sum
   float* st_a = st_l + group;          // [group] rescale factor of this chunk
 
-  const int n_out = group * d;
-  for (int i = tid; i < n_out; i += AG_THREADS)
+  const int n_out = group * dv;
+  for (int i = tid; i < group * d; i += AG_THREADS)
     qs[i] = to_f32<T>(q[(size_t)t * q_stride + (size_t)g * group * d + i]);
   if (tid < group) {
     st_m[tid] = -INFINITY;
@@ -56,16 +60,18 @@ __global__ __launch_bounds__(AG_THREADS) void paged_attention_generic_kernel(
     for (int i = tid; i < CH * d; i += AG_THREADS) {
       const int j = i / d, e = i % d;
       const int kp = c0 + j;
-      float kv = 0.f, vv = 0.f;
-      if (kp >= lo && kp <= pos) {
-        const int page = table[kp / P];
-        const int p = kp % P;
-        const size_t base = ((size_t)page * nkv + g) * P * d;
-        kv = to_f32<T>(kcache[base + key_offset(P, p, e)]);
-        vv = to_f32<T>(vcache[base + value_offset(d, p, e)]);
-      }
+      float kv = 0.f;
+      if (kp >= lo && kp <= pos)
+        kv = to_f32<T>(kcache[((size_t)table[kp / P] * nkv + g) * P * d + key_offset(P, kp % P, e)]);
       Ks[j * (d + 1) + e] = kv;
-      Vs[j * d + e] = vv;
+    }
+    for (int i = tid; i < CH * dv; i += AG_THREADS) {
+      const int j = i / dv, e = i % dv;
+      const int kp = c0 + j;
+      float vv = 0.f;
+      if (kp >= lo && kp <= pos)
+        vv = to_f32<T>(vcache[((size_t)table[kp / P] * nkv + g) * P * dv + value_offset(dv, kp % P, e)]);
+      Vs[j * dv + e] = vv;
     }
     __syncthreads();
     // scores
@@ -104,10 +110,10 @@ __global__ __launch_bounds__(AG_THREADS) void paged_attention_generic_kernel(
     for (int r = 0; r < AG_MAX_ACC; ++r) {
       const int i = tid + r * AG_THREADS;
       if (i < n_out) {
-        const int gq = i / d, e = i % d;
+        const int gq = i / dv, e = i % dv;
         float a = acc[r] * st_a[gq];
         const float* pv = Ss + gq * CH;
-        for (int j = 0; j < CH; ++j) a = fmaf(pv[j], Vs[j * d + e], a);
+        for (int j = 0; j < CH; ++j) a = fmaf(pv[j], Vs[j * dv + e], a);
         acc[r] = a;
       }
     }
@@ -117,14 +123,22 @@ __global__ __launch_bounds__(AG_THREADS) void paged_attention_generic_kernel(
   for (int r = 0; r < AG_MAX_ACC; ++r) {
     const int i = tid + r * AG_THREADS;
     if (i < n_out) {
-      const int gq = i / d;
-      out[(size_t)t * out_stride + (size_t)g * group * d + i] = from_f32<T>(acc[r] / st_l[gq]);
+      const int gq = i / dv;
+      float a = acc[r], l = st_l[gq];
+      if (sink) {
+        // the sink joins the softmax like one more score: the maximum may rise to it
+        const float sk = sink[g * group + gq], m = st_m[gq], m_all = fmaxf(m, sk);
+        const float keep = expf(m - m_all);
+        a *= keep;
+        l = l * keep + expf(sk - m_all);
+      }
+      out[(size_t)t * out_stride + (size_t)g * group * dv + i] = from_f32<T>(a / l);
     }
   }
 }
 
-static size_t ag_smem_bytes(int group, int d, int ch) {
-  return sizeof(float) * ((size_t)group * d + (size_t)ch * (d + 1) + (size_t)ch * d +
+static size_t ag_smem_bytes(int group, int d, int dv, int ch) {
+  return sizeof(float) * ((size_t)group * d + (size_t)ch * (d + 1) + (size_t)ch * dv +
                           (size_t)group * ch + 3 * (size_t)group);
 }
 
@@ -132,22 +146,22 @@ template <typename T, int CH>
 static void ag_launch(const void* q, int q_stride, void* out, int out_stride, const void* kcache,
                       const void* vcache, const int* block_table, int table_stride,
                       const int* token_req, const int* positions, int n_tokens, int nq, int nkv,
-                      int d, int P, int window, float scale, hipStream_t stream) {
+                      int d, int dv, int P, int window, float scale, const float* sink, hipStream_t stream) {
   hipLaunchKernelGGL((paged_attention_generic_kernel<T, CH>), dim3(n_tokens, nkv),
-                     dim3(AG_THREADS), ag_smem_bytes(nq / nkv, d, CH), stream, (const T*)q,
+                     dim3(AG_THREADS), ag_smem_bytes(nq / nkv, d, dv, CH), stream, (const T*)q,
                      q_stride, (T*)out, out_stride, (const T*)kcache, (const T*)vcache,
-                     block_table, table_stride, token_req, positions, nq, nkv, d, P, window, scale);
+                     block_table, table_stride, token_req, positions, nq, nkv, d, dv, P, window, scale, sink);
 }
 
 // Whether the kernel takes this group and head size at all (0 and the reason in tk_last_error
 // when not): asked when a cache is made, so that a model is refused before its first step.
-TK_API int tk_paged_attention_generic_fits(int nq, int nkv, int d) {
-  TK_REQUIRE(nq > 0 && nkv > 0 && d > 0 && nq % nkv == 0, "paged_attention: bad sizes nq=%d nkv=%d d=%d", nq, nkv, d);
+TK_API int tk_paged_attention_generic_fits(int nq, int nkv, int d, int dv) {
+  TK_REQUIRE(nq > 0 && nkv > 0 && d > 0 && dv > 0 && nq % nkv == 0, "paged_attention: bad sizes nq=%d nkv=%d d=%d dv=%d", nq, nkv, d, dv);
   const int group = nq / nkv;
-  TK_REQUIRE(group * d <= AG_THREADS * AG_MAX_ACC,
-             "paged_attention: group %d x head size %d exceeds %d outputs per kv head", group, d,
+  TK_REQUIRE(group * dv <= AG_THREADS * AG_MAX_ACC,
+             "paged_attention: group %d x value size %d exceeds %d outputs per kv head", group, dv,
              AG_THREADS * AG_MAX_ACC);
-  TK_REQUIRE(ag_smem_bytes(group, d, 8) <= 64 * 1024,
+  TK_REQUIRE(ag_smem_bytes(group, d, dv, 8) <= 64 * 1024,
              "paged_attention: head size %d with group %d does not fit the local memory", d, group);
   return 0;
 }
@@ -156,26 +170,26 @@ TK_API int tk_paged_attention_generic(int dt, const void* q, int q_stride, void*
                                           int out_stride, const void* kcache, const void* vcache,
                                           const int* block_table, int table_stride,
                                           const int* token_req, const int* positions, int n_tokens,
-                                          int nq, int nkv, int d, int P, int window, float scale,
-                                          hipStream_t stream) {
-  TK_REQUIRE(n_tokens >= 0 && nq > 0 && nkv > 0 && d > 0 && P > 0 && nq % nkv == 0,
-             "paged_attention: bad sizes tokens=%d nq=%d nkv=%d d=%d P=%d", n_tokens, nq, nkv, d,
+                                          int nq, int nkv, int d, int dv, int P, int window, float scale,
+                                          const float* sink, hipStream_t stream) {
+  TK_REQUIRE(n_tokens >= 0 && nq > 0 && nkv > 0 && d > 0 && dv > 0 && P > 0 && nq % nkv == 0,
+             "paged_attention: bad sizes tokens=%d nq=%d nkv=%d d=%d dv=%d P=%d", n_tokens, nq, nkv, d, dv,
              P);
   const int group = nq / nkv;
-  TK_REQUIRE(group * d <= AG_THREADS * AG_MAX_ACC,
-             "paged_attention: group %d x head size %d exceeds %d outputs per kv head", group, d,
+  TK_REQUIRE(group * dv <= AG_THREADS * AG_MAX_ACC,
+             "paged_attention: group %d x value size %d exceeds %d outputs per kv head", group, dv,
              AG_THREADS * AG_MAX_ACC);
-  TK_REQUIRE(q_stride >= nq * d && out_stride >= nq * d, "paged_attention: row strides too short");
+  TK_REQUIRE(q_stride >= nq * d && out_stride >= nq * dv, "paged_attention: row strides too short");
   TK_REQUIRE(nkv < 65536, "paged_attention: too many kv heads");
   if (n_tokens == 0) return 0;
   const size_t limit = 64 * 1024;
   int ch = 64;
-  while (ch > 8 && ag_smem_bytes(group, d, ch) > limit) ch /= 2;
-  TK_REQUIRE(ag_smem_bytes(group, d, ch) <= limit,
+  while (ch > 8 && ag_smem_bytes(group, d, dv, ch) > limit) ch /= 2;
+  TK_REQUIRE(ag_smem_bytes(group, d, dv, ch) <= limit,
              "paged_attention: head size %d with group %d does not fit the local memory", d, group);
 #define AG_CASE(T, CHV)                                                                         \
   ag_launch<T, CHV>(q, q_stride, out, out_stride, kcache, vcache, block_table, table_stride,    \
-                    token_req, positions, n_tokens, nq, nkv, d, P, window, scale, stream)
+                    token_req, positions, n_tokens, nq, nkv, d, dv, P, window, scale, sink, stream)
   if (dt == TK_F32) {
     if (ch == 64) AG_CASE(float, 64);
     else if (ch == 32) AG_CASE(float, 32);

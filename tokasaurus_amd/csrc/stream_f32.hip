@@ -1,0 +1,111 @@
+// Kernels for models whose residual stream is kept in 32-bit whatever the storage type of
+// the weights: a scaled embedding that writes 32-bit rows, the residual update
+//     x <- x + mult * (a + b)
+// of a block whose branches run side by side, fused with the RMS norms that read the new
+// stream (one statistic, up to two weight vectors), and the soft cap of the logits.
+// T is the storage type of the normed rows that the next products read.
+#include "common.h"
+
+// --------------------------------------------------------------------------
+// out[t, :] = float(table[id_t, :]) * scale; id_t < 0 names slot -id_t-1 of `last_token`.
+// --------------------------------------------------------------------------
+template <typename T>
+__global__ void embed_scaled_kernel(const int* __restrict__ ids, const int* __restrict__ last_token,
+                                    const T* __restrict__ table, float* __restrict__ out, int hidden,
+                                    int vocab, float scale) {
+  const int t = blockIdx.x;
+  int id = ids[t];
+  if (id < 0) id = last_token[-id - 1];
+  id = min(max(id, 0), vocab - 1);
+  const T* src = table + (size_t)id * hidden;
+  float* dst = out + (size_t)t * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_f32<T>(src[i]) * scale;
+}
+
+TK_API int tk_embed_scaled(int dt, const int* ids, const int* last_token, const void* table,
+                           float* out, int n_tokens, int hidden, int vocab, float scale,
+                           hipStream_t stream) {
+  TK_REQUIRE(n_tokens >= 0 && hidden > 0 && vocab > 0, "embed_scaled: bad sizes %d %d %d", n_tokens,
+             hidden, vocab);
+  if (n_tokens == 0) return 0;
+  if (dt == TK_F32)
+    hipLaunchKernelGGL(embed_scaled_kernel<float>, dim3(n_tokens), dim3(256), 0, stream, ids,
+                       last_token, (const float*)table, out, hidden, vocab, scale);
+  else
+    hipLaunchKernelGGL(embed_scaled_kernel<bf16_t>, dim3(n_tokens), dim3(256), 0, stream, ids,
+                       last_token, (const bf16_t*)table, out, hidden, vocab, scale);
+  TK_CHECK_LAUNCH("embed_scaled");
+  return 0;
+}
+
+// --------------------------------------------------------------------------
+// One row a workgroup.  Reads x (32-bit) and the branches a, b (32-bit, either may be null),
+// writes x_out = x + mult * (a + b) (32-bit; may be x itself; null when there is no branch and
+// the stream stays as it is) and, for each of up to two norms, the row
+//     x_out / sqrt(mean(x_out^2) + eps) * (offset + w)
+// rounded once to T.  `offset` is 1 for weights stored around zero, 0 for plain ones.
+// Norm weights are 32-bit.
+// --------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void residual_norm_kernel(
+    const float* __restrict__ x, const float* __restrict__ a, const float* __restrict__ b, float mult,
+    float* x_out, const float* __restrict__ w1, const float* __restrict__ w2, float offset, float eps,
+    T* __restrict__ h1, T* __restrict__ h2, int hidden) {
+  __shared__ float red[16];
+  const size_t row = (size_t)blockIdx.x * hidden;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    float v = x[row + i];
+    if (a || b) {
+      float y = a ? a[row + i] : 0.f;
+      if (b) y += b[row + i];
+      v = fmaf(mult, y, v);
+      x_out[row + i] = v;
+    }
+    ss = fmaf(v, v, ss);
+  }
+  if (!w1 && !w2) return;
+  ss = block_sum(ss, red);
+  const float rstd = 1.0f / sqrtf(ss / (float)hidden + eps);
+  const float* src = (a || b) ? x_out : x;  // a thread reads back what it wrote
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    const float n = src[row + i] * rstd;
+    if (w1) h1[row + i] = from_f32<T>(n * (offset + w1[i]));
+    if (w2) h2[row + i] = from_f32<T>(n * (offset + w2[i]));
+  }
+}
+
+TK_API int tk_residual_norm(int dt, const float* x, const float* a, const float* b, float mult,
+                            float* x_out, const float* w1, const float* w2, float offset, float eps,
+                            void* h1, void* h2, int rows, int hidden, hipStream_t stream) {
+  TK_REQUIRE(rows >= 0 && hidden > 0, "residual_norm: bad sizes %d %d", rows, hidden);
+  TK_REQUIRE(!(a || b) || x_out, "residual_norm: a branch needs a place for the new stream");
+  TK_REQUIRE((!w1 || h1) && (!w2 || h2), "residual_norm: a norm needs a place for its rows");
+  if (rows == 0) return 0;
+  if (dt == TK_F32)
+    hipLaunchKernelGGL(residual_norm_kernel<float>, dim3(rows), dim3(256), 0, stream, x, a, b, mult,
+                       x_out, w1, w2, offset, eps, (float*)h1, (float*)h2, hidden);
+  else
+    hipLaunchKernelGGL(residual_norm_kernel<bf16_t>, dim3(rows), dim3(256), 0, stream, x, a, b, mult,
+                       x_out, w1, w2, offset, eps, (bf16_t*)h1, (bf16_t*)h2, hidden);
+  TK_CHECK_LAUNCH("residual_norm");
+  return 0;
+}
+
+// --------------------------------------------------------------------------
+// logits <- cap * tanh(logits / cap), in place, 32-bit.
+// --------------------------------------------------------------------------
+__global__ void softcap_kernel(float* __restrict__ v, size_t n, float cap) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) v[i] = cap * tanhf(v[i] / cap);
+}
+
+TK_API int tk_softcap(float* v, size_t n, float cap, hipStream_t stream) {
+  TK_REQUIRE(cap > 0.f, "softcap: the cap must be positive");
+  if (n == 0) return 0;
+  const size_t blocks = (n + 255) / 256;
+  TK_REQUIRE(blocks < (1u << 31), "softcap: too many values");
+  hipLaunchKernelGGL(softcap_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, v, n, cap);
+  TK_CHECK_LAUNCH("softcap");
+  return 0;
+}

@@ -34,10 +34,18 @@ _SIGNATURES: dict[str, dict[str, list]] = {
         "tk_add_bias": [c_int, _P, _P, c_int, c_int, _P],
         "tk_head_rmsnorm": [c_int, _P, c_int, _P, c_int, c_int, c_int, c_int, c_int, c_float, _P],
         "tk_paged_attention_generic": [c_int, _P, c_int, _P, c_int, _P, _P, _P, c_int, _P, _P]
-        + [c_int] * 6
-        + [c_float, _P],
-        "tk_paged_attention_generic_fits": [c_int, c_int, c_int],
+        + [c_int] * 7
+        + [c_float, _P, _P],
+        "tk_paged_attention_generic_fits": [c_int, c_int, c_int, c_int],
         "tk_add": [c_int, _P, _P, _P, c_size_t, _P],
+        "tk_embed_scaled": [c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_float, _P],
+        "tk_residual_norm": [c_int, _P, _P, _P, c_float, _P, _P, _P, c_float, c_float, _P, _P, c_int, c_int, _P],
+        "tk_softcap": [_P, c_size_t, c_float, _P],
+        "tk_qk_prepare": [c_int, _P, c_int, _P, _P, _P, c_int, _P, _P, c_float, _P, _P, _P] + [c_int] * 8 + [_P],
+        "tk_delta_prepare": [c_int, _P, c_int, c_int, _P, _P, c_int, _P, _P, _P, c_size_t, c_size_t, _P, _P, _P, _P]
+        + [c_int] * 7 + [_P],
+        "tk_delta_rule": [_P, c_int, _P, c_size_t, _P, _P, _P] + [c_int] * 6 + [_P],
+        "tk_gated_head_norm": [c_int, _P, _P, _P, c_float, _P, c_int, c_int, c_int, _P],
         "tk_sample": [_P, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P],
         "tk_sample_static": [_P, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P],
         "tk_sample_chunks": [c_int],

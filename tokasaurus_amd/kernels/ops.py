@@ -66,13 +66,16 @@ def value_pages_shape(pages: int, nkv: int, page_size: int, head_dim: int) -> tu
     return (pages, nkv, page_size // VALUE_QUAD, head_dim, VALUE_QUAD)
 
 
-def _check_pages(kcache: torch.Tensor, vcache: torch.Tensor, nkv: int, page_size: int, head_dim: int, dtype: torch.dtype, who: str) -> None:
+def _check_pages(kcache: torch.Tensor, vcache: torch.Tensor, nkv: int, page_size: int, head_dim: int, dtype: torch.dtype, who: str,
+                 value_dim: int | None = None) -> None:
+    """``value_dim``: the size of a value head where it differs from a key head's."""
     pages = kcache.shape[0]
+    vd = head_dim if value_dim is None else value_dim
     # (the shapes are compared in place: this runs twice a layer of an eager step)
     if (kcache.shape != (pages, nkv, head_dim // KEY_PIECE, page_size, KEY_PIECE) or head_dim % KEY_PIECE or not kcache.is_contiguous()):
         raise KernelError(f"{who}: key pages must be contiguous {key_pages_shape(pages, nkv, page_size, head_dim)}, got {tuple(kcache.shape)}")
-    if (vcache.shape != (pages, nkv, page_size // VALUE_QUAD, head_dim, VALUE_QUAD) or page_size % VALUE_QUAD or not vcache.is_contiguous()):
-        raise KernelError(f"{who}: value pages must be contiguous {value_pages_shape(pages, nkv, page_size, head_dim)}, got {tuple(vcache.shape)}")
+    if (vcache.shape != (pages, nkv, page_size // VALUE_QUAD, vd, VALUE_QUAD) or page_size % VALUE_QUAD or not vcache.is_contiguous()):
+        raise KernelError(f"{who}: value pages must be contiguous {value_pages_shape(pages, nkv, page_size, vd)}, got {tuple(vcache.shape)}")
     if kcache.dtype != dtype or vcache.dtype != dtype:
         raise KernelError(f"{who}: the cache must be {dtype}")
 
@@ -348,10 +351,18 @@ def paged_attention_generic(
     page_size: int,
     window: int = 0,
     scale: float | None = None,
+    value_dim: int | None = None,
+    sink: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """Attention of every token over its request's pages (see rope_append for
-    the page layout).  ``q`` is 2-d, its first nq*d columns are the query heads."""
-    _gpu(q, kcache, vcache, block_table, token_req, positions)
+    the page layout).  ``q`` is 2-d, its first nq*d columns are the query heads.
+    ``value_dim``: the size of a value head (a key head's by default); the result is
+    [tokens, nq * value_dim].  ``sink`` (32-bit, one number a query head): exp(sink) joins the
+    softmax's denominator once, with no key and no value."""
+    _gpu(q, kcache, vcache, block_table, token_req, positions, sink)
+    vd = head_dim if value_dim is None else int(value_dim)
+    _need(sink is None or (sink.shape == (nq,) and sink.dtype == torch.float32 and sink.is_contiguous()),
+          f"attention: the sinks must be contiguous float32 [{nq}]")
     _need(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= nq * head_dim,
           "attention: q must be 2-d with unit inner stride and nq*d leading columns")
     n = q.shape[0]
@@ -360,8 +371,8 @@ def paged_attention_generic(
     _i32(positions, "positions")
     _need(block_table.dim() == 2, "block_table must be [requests, width]")
     _need(positions.numel() == n and token_req.numel() == n, "positions/token_req must have one entry a token")
-    _check_pages(kcache, vcache, nkv, page_size, head_dim, q.dtype, "attention")
-    out = torch.empty((n, nq * head_dim), dtype=q.dtype, device=q.device)
+    _check_pages(kcache, vcache, nkv, page_size, head_dim, q.dtype, "attention", vd)
+    out = torch.empty((n, nq * vd), dtype=q.dtype, device=q.device)
     call(
         "tk_paged_attention_generic",
         dtype_code(q.dtype),
@@ -379,9 +390,11 @@ def paged_attention_generic(
         nq,
         nkv,
         head_dim,
+        vd,
         page_size,
         int(window),
         float(scale if scale is not None else 1.0 / math.sqrt(head_dim)),
+        sink.data_ptr() if sink is not None else None,
         _stream(),
     )
     return out
@@ -393,14 +406,17 @@ def attention_mfma_supports(dtype: torch.dtype, head_dim: int, page_size: int) -
             and page_size >= 4 and page_size & (page_size - 1) == 0)
 
 
-def check_attention_shape(dtype: torch.dtype, nq: int, nkv: int, head_dim: int, page_size: int) -> None:
+def check_attention_shape(dtype: torch.dtype, nq: int, nkv: int, head_dim: int, page_size: int,
+                          value_dim: int | None = None, generic_only: bool = False) -> None:
     """Refuse, with the kernel's own reason, head counts and sizes that neither attention
     kernel takes for this storage type and page size.  Called when a cache is made for a
-    mixer, so that a model that cannot run is refused before its first step."""
+    mixer, so that a model that cannot run is refused before its first step.  ``generic_only``:
+    the mixer uses what only the 32-bit-arithmetic kernel has (a value size of its own, sinks)."""
+    vd = head_dim if value_dim is None else value_dim
     key_pages_shape(1, nkv, page_size, head_dim)
-    value_pages_shape(1, nkv, page_size, head_dim)
-    if not attention_mfma_supports(dtype, head_dim, page_size):
-        call("tk_paged_attention_generic_fits", nq, nkv, head_dim)
+    value_pages_shape(1, nkv, page_size, vd)
+    if generic_only or vd != head_dim or not attention_mfma_supports(dtype, head_dim, page_size):
+        call("tk_paged_attention_generic_fits", nq, nkv, head_dim, vd)
 
 
 ATTENTION_GROUP = 4  # wavefronts (of two neighbouring row tiles each) in a workgroup of the grouped prompt kernel
@@ -1056,3 +1072,235 @@ def publish_step(host_ring: torch.Tensor, counter: torch.Tensor, ids: torch.Tens
     call("tk_publish_step", host_ring.data_ptr(), counter.data_ptr(), host_ring.shape[0], host_ring.shape[1], ids.data_ptr(),
          logprobs.data_ptr() if logprobs is not None else None, rows,
          topk_ids.data_ptr() if k else None, topk_logprobs.data_ptr() if k else None, k, _stream())
+
+
+# --------------------------------------------------------------------------
+# a residual stream kept in 32-bit
+# --------------------------------------------------------------------------
+
+def _f32_vector(t: torch.Tensor | None, n: int, name: str) -> None:
+    if t is not None and (t.shape != (n,) or t.dtype != torch.float32 or not t.is_contiguous()):
+        raise KernelError(f"{name} must be contiguous float32 [{n}]")
+
+
+def embed_scaled(ids: torch.Tensor, table: torch.Tensor, scale: float, last_token: torch.Tensor | None = None) -> torch.Tensor:
+    """out[t] = float32(table[ids[t]]) * scale: the first rows of a 32-bit residual stream;
+    ids[t] < 0 reads the token from last_token[-ids[t]-1]."""
+    _gpu(ids, table, last_token)
+    _i32(ids, "ids")
+    _need(table.dim() == 2 and table.is_contiguous(), "embedding table must be contiguous [V, H]")
+    if last_token is not None:
+        _i32(last_token, "last_token")
+    n = ids.numel()
+    vocab, hidden = table.shape
+    out = torch.empty((n, hidden), dtype=torch.float32, device=table.device)
+    call("tk_embed_scaled", dtype_code(table.dtype), ids.data_ptr(), last_token.data_ptr() if last_token is not None else None,
+         table.data_ptr(), out.data_ptr(), n, hidden, vocab, float(scale), _stream())
+    return out
+
+
+def residual_norm(
+    x: torch.Tensor,
+    branches: tuple[torch.Tensor | None, torch.Tensor | None] = (None, None),
+    mult: float = 1.0,
+    weights: tuple[torch.Tensor | None, torch.Tensor | None] = (None, None),
+    unit_offset: bool = False,
+    eps: float = 0.0,
+    out_dtype: torch.dtype = torch.float32,
+    in_place: bool = True,
+) -> tuple[torch.Tensor, torch.Tensor | None, torch.Tensor | None]:
+    """The update of a 32-bit residual stream and the norms that read the new stream, in one pass:
+    ``x_new = x + mult * (a + b)`` for the 32-bit ``branches`` (either may be None; with neither
+    the stream stays), then for each of up to two 32-bit ``weights`` the rows
+    ``x_new / sqrt(mean(x_new^2) + eps) * (w + (1 if unit_offset else 0))`` rounded once to
+    ``out_dtype``.  Returns (x_new, normed rows for weights[0], for weights[1]).  ``in_place``:
+    the new stream overwrites ``x``."""
+    a, b = branches
+    w1, w2 = weights
+    _gpu(x, a, b, w1, w2)
+    _need(x.dim() == 2 and x.dtype == torch.float32 and x.is_contiguous(), "residual_norm: the stream must be contiguous float32 [rows, H]")
+    rows, hidden = x.shape
+    for y in (a, b):
+        _need(y is None or (y.shape == x.shape and y.dtype == torch.float32 and y.is_contiguous()),
+              "residual_norm: a branch must be contiguous float32 of the stream's shape")
+    _f32_vector(w1, hidden, "residual_norm: a norm weight")
+    _f32_vector(w2, hidden, "residual_norm: a norm weight")
+    changed = a is not None or b is not None
+    x_out = (x if in_place else torch.empty_like(x)) if changed else x
+    h1 = torch.empty((rows, hidden), dtype=out_dtype, device=x.device) if w1 is not None else None
+    h2 = torch.empty((rows, hidden), dtype=out_dtype, device=x.device) if w2 is not None else None
+    if rows == 0:
+        return x_out, h1, h2
+    call("tk_residual_norm", dtype_code(out_dtype), x.data_ptr(), a.data_ptr() if a is not None else None,
+         b.data_ptr() if b is not None else None, float(mult), x_out.data_ptr() if changed else None,
+         w1.data_ptr() if w1 is not None else None, w2.data_ptr() if w2 is not None else None,
+         1.0 if unit_offset else 0.0, float(eps), h1.data_ptr() if h1 is not None else None,
+         h2.data_ptr() if h2 is not None else None, rows, hidden, _stream())
+    return x_out, h1, h2
+
+
+def softcap_(logits: torch.Tensor, cap: float) -> torch.Tensor:
+    """logits <- cap * tanh(logits / cap), in place (contiguous float32)."""
+    _gpu(logits)
+    _need(logits.dtype == torch.float32 and logits.is_contiguous(), "softcap: logits must be contiguous float32")
+    call("tk_softcap", logits.data_ptr(), logits.numel(), float(cap), _stream())
+    return logits
+
+
+# --------------------------------------------------------------------------
+# attention with norms over the whole projection and a rotation of neighbouring elements
+# --------------------------------------------------------------------------
+
+def qk_prepare(
+    qkv: torch.Tensor,
+    positions: torch.Tensor,
+    token_req: torch.Tensor,
+    block_table: torch.Tensor | None,
+    q_weight: torch.Tensor | None,
+    k_weight: torch.Tensor | None,
+    eps: float,
+    freq: torch.Tensor | None,
+    kcache: torch.Tensor | None,
+    vcache: torch.Tensor | None,
+    nq: int,
+    nkv: int,
+    key_dim: int,
+    value_dim: int,
+    page_size: int,
+    write_cache: bool = True,
+) -> None:
+    """In place on the rows [q: nq*dk | k: nkv*dk | v: nkv*dv] (only q when not ``write_cache``):
+    the RMS norm of the whole query row and of the whole key row (32-bit weights of those sizes,
+    or None for no norm), the rotation of elements (2i, 2i+1) of every head by position *
+    freq[i] for i < len(freq), and the append of keys and values to the token's page."""
+    _gpu(qkv, positions, token_req, block_table, q_weight, k_weight, freq, kcache, vcache)
+    _need(qkv.dim() == 2 and qkv.stride(1) == 1, "qk_prepare: rows must be 2-d with unit inner stride")
+    n = qkv.shape[0]
+    need = nq * key_dim + (nkv * (key_dim + value_dim) if write_cache else 0)
+    _need(qkv.shape[1] >= need, f"qk_prepare: rows of {qkv.shape[1]} hold no {need} elements")
+    _i32(positions, "positions")
+    _i32(token_req, "token_req")
+    _need(positions.numel() == n and token_req.numel() == n, "positions/token_req must have one entry a token")
+    _f32_vector(q_weight, nq * key_dim, "qk_prepare: the query norm's weight")
+    _f32_vector(k_weight, nkv * key_dim, "qk_prepare: the key norm's weight")
+    rot = 0
+    if freq is not None:
+        _need(freq.dim() == 1 and freq.dtype == torch.float32 and freq.is_contiguous() and 2 * freq.numel() <= key_dim,
+              "qk_prepare: frequencies must be contiguous float32, at most half a head's size of them")
+        rot = 2 * freq.numel()
+    if write_cache:
+        _i32(block_table, "block_table")
+        _need(block_table.dim() == 2, "block_table must be [requests, width]")
+        _check_pages(kcache, vcache, nkv, page_size, key_dim, qkv.dtype, "qk_prepare", value_dim)
+    call("tk_qk_prepare", dtype_code(qkv.dtype), qkv.data_ptr(), qkv.stride(0), positions.data_ptr(), token_req.data_ptr(),
+         block_table.data_ptr() if write_cache else None, block_table.stride(0) if write_cache else 0,
+         q_weight.data_ptr() if q_weight is not None else None, k_weight.data_ptr() if k_weight is not None else None,
+         float(eps), freq.data_ptr() if freq is not None else None,
+         kcache.data_ptr() if write_cache else None, vcache.data_ptr() if write_cache else None,
+         n, nq, nkv if write_cache else 0, key_dim, value_dim, rot, page_size, 1 if write_cache else 0, _stream())
+
+
+# --------------------------------------------------------------------------
+# the gated delta rule with a decay per key channel
+# --------------------------------------------------------------------------
+
+def delta_state_size(heads: int, kv_heads: int, key_dim: int, value_dim: int, taps: int) -> int:
+    """32-bit numbers a request keeps for one such mixer: the matrices S and the convolutions' tails."""
+    return heads * key_dim * value_dim + (taps - 1) * (2 * kv_heads * key_dim + heads * value_dim)
+
+
+def delta_rec_width(heads: int, kv_heads: int, key_dim: int, value_dim: int) -> int:
+    return 2 * kv_heads * key_dim + heads * value_dim + heads * key_dim + heads
+
+
+def delta_prepare(
+    proj: torch.Tensor,
+    col_b: int,
+    a_pre: torch.Tensor,
+    conv_w: torch.Tensor,
+    a_log: torch.Tensor,
+    dt_bias: torch.Tensor,
+    state: torch.Tensor,
+    q_start: torch.Tensor,
+    token_req: torch.Tensor,
+    slots: torch.Tensor,
+    heads: int,
+    kv_heads: int,
+    key_dim: int,
+    value_dim: int,
+) -> torch.Tensor:
+    """What the recurrence reads, in 32-bit [tokens, q | k | v | decay | beta]: the rows
+    ``proj`` [q | k | v | ...] pass their short causal convolutions (``conv_w`` [channels, taps],
+    earlier inputs from this step's rows or the tail in the request's ``state`` row) and silu; q
+    and k become unit vectors per head (q also times key_dim^-1/2); decay = exp(-exp(a_log) *
+    softplus(a_pre + dt_bias)); beta = sigmoid(proj[:, col_b + head]).  The tails in ``state``
+    are then moved on by this step's rows."""
+    _gpu(proj, a_pre, conv_w, a_log, dt_bias, state, q_start, token_req, slots)
+    n = proj.shape[0]
+    channels = 2 * kv_heads * key_dim + heads * value_dim
+    _need(proj.dim() == 2 and proj.stride(1) == 1 and proj.dtype in _DT, "delta_prepare: rows must be 2-d with unit inner stride")
+    _need(conv_w.dim() == 2 and conv_w.shape[0] == channels and conv_w.dtype == torch.float32 and conv_w.is_contiguous(),
+          f"delta_prepare: the convolutions' weights must be contiguous float32 [{channels}, taps]")
+    taps = conv_w.shape[1]
+    _need(a_pre.shape == (n, heads * key_dim) and a_pre.dtype == torch.float32 and a_pre.is_contiguous(),
+          "delta_prepare: the decay's projection must be contiguous float32 [tokens, heads * key_dim]")
+    _f32_vector(a_log, heads, "delta_prepare: a_log")
+    _f32_vector(dt_bias, heads * key_dim, "delta_prepare: dt_bias")
+    _need(state.dim() == 2 and state.dtype == torch.float32 and state.is_contiguous()
+          and state.shape[1] >= delta_state_size(heads, kv_heads, key_dim, value_dim, taps), "delta_prepare: state rows too short")
+    for t, name in ((q_start, "q_start"), (token_req, "token_req"), (slots, "slots")):
+        _i32(t, name)
+    _need(token_req.numel() == n and q_start.numel() == slots.numel() + 1, "delta_prepare: one request a token, one slot a request")
+    width = delta_rec_width(heads, kv_heads, key_dim, value_dim)
+    rec = torch.empty((n, width), dtype=torch.float32, device=proj.device)
+    call("tk_delta_prepare", dtype_code(proj.dtype), proj.data_ptr(), proj.stride(0), int(col_b), a_pre.data_ptr(),
+         conv_w.data_ptr(), taps, a_log.data_ptr(), dt_bias.data_ptr(), state.data_ptr(), state.stride(0),
+         heads * key_dim * value_dim, q_start.data_ptr(), token_req.data_ptr(), slots.data_ptr(), rec.data_ptr(), width,
+         n, slots.numel(), heads, kv_heads, key_dim, value_dim, _stream())
+    return rec
+
+
+def delta_rule_columns(requests: int, heads: int, key_dim: int, value_dim: int) -> int:
+    """Value columns a workgroup of the recurrence owns: as many as still leave the chip a few
+    workgroups a compute unit (a column's arithmetic does not depend on the choice)."""
+    most = 128 if key_dim <= 128 else 32
+    cols = 8
+    while cols * 2 <= most and cols < value_dim and requests * heads * -(-value_dim // (cols * 2)) >= 1024:
+        cols *= 2
+    return cols
+
+
+def delta_rule(rec: torch.Tensor, state: torch.Tensor, q_start: torch.Tensor, slots: torch.Tensor,
+               heads: int, kv_heads: int, key_dim: int, value_dim: int) -> torch.Tensor:
+    """The recurrence over every request's tokens of this step, from and to the matrices in the
+    requests' ``state`` rows: o [tokens, heads * value_dim] in 32-bit."""
+    _gpu(rec, state, q_start, slots)
+    n = rec.shape[0]
+    _need(rec.dim() == 2 and rec.dtype == torch.float32 and rec.is_contiguous()
+          and rec.shape[1] == delta_rec_width(heads, kv_heads, key_dim, value_dim), "delta_rule: rows of the wrong width")
+    _need(state.dim() == 2 and state.dtype == torch.float32 and state.is_contiguous()
+          and state.shape[1] >= heads * key_dim * value_dim, "delta_rule: state rows too short")
+    _i32(q_start, "q_start")
+    _i32(slots, "slots")
+    _need(q_start.numel() == slots.numel() + 1, "delta_rule: one slot a request")
+    o = torch.empty((n, heads * value_dim), dtype=torch.float32, device=rec.device)
+    cols = delta_rule_columns(slots.numel(), heads, key_dim, value_dim)
+    call("tk_delta_rule", rec.data_ptr(), rec.stride(0), state.data_ptr(), state.stride(0), q_start.data_ptr(),
+         slots.data_ptr(), o.data_ptr(), slots.numel(), heads, kv_heads, key_dim, value_dim, cols, _stream())
+    return o
+
+
+def gated_head_norm(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps: float, heads: int, value_dim: int,
+                    out_dtype: torch.dtype) -> torch.Tensor:
+    """Every head's ``value_dim`` numbers divided by their root mean square, times ``weight``
+    [value_dim], times sigmoid(gate); 32-bit in, rounded once to ``out_dtype``."""
+    _gpu(o, gate, weight)
+    n = o.shape[0]
+    for t in (o, gate):
+        _need(t.shape == (n, heads * value_dim) and t.dtype == torch.float32 and t.is_contiguous(),
+              "gated_head_norm: inputs must be contiguous float32 [tokens, heads * value_dim]")
+    _f32_vector(weight, value_dim, "gated_head_norm: the weight")
+    out = torch.empty((n, heads * value_dim), dtype=out_dtype, device=o.device)
+    call("tk_gated_head_norm", dtype_code(out_dtype), o.data_ptr(), gate.data_ptr(), weight.data_ptr(), float(eps),
+         out.data_ptr(), n, heads, value_dim, _stream())
+    return out

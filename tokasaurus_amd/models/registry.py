@@ -11,6 +11,8 @@ from typing import Any, Callable
 
 from tokasaurus_amd.config.model_config import ConfigError, LlamaConfig, read_config_json
 from tokasaurus_amd.models.causal_lm import CausalLM
+from tokasaurus_amd.config.kupuzen_config import KupuzenConfig
+from tokasaurus_amd.models.kupuzen import kupuzen_spec
 from tokasaurus_amd.models.llama import llama_spec
 from tokasaurus_amd.models.spec import ModelSpec
 
@@ -35,6 +37,7 @@ def register_architecture(arch: Architecture, replace: bool = False) -> None:
 
 
 register_architecture(Architecture("llama", LlamaConfig.from_dict, llama_spec, class_names=("LlamaForCausalLM",)))
+register_architecture(Architecture("kupuzen", KupuzenConfig.from_dict, kupuzen_spec, class_names=("Kupuzen",)))
 
 
 def architecture_of(config_dict: dict[str, Any]) -> Architecture:
@@ -43,7 +46,9 @@ def architecture_of(config_dict: dict[str, Any]) -> Architecture:
     architecture claims."""
     name = config_dict.get("model_type")
     if name is None:
-        classes = config_dict.get("architectures") or []
+        # a file may name its one class under "architecture" instead of listing classes
+        one = config_dict.get("architecture")
+        classes = list(config_dict.get("architectures") or []) + ([one] if isinstance(one, str) else [])
         by_class = {c: a for a in ARCHITECTURES.values() for c in a.class_names}
         for c in classes:
             if c in by_class:
@@ -62,6 +67,11 @@ def config_from_folder(model_dir: str | Path, rope_scaling_override: tuple[bool,
     cfg = arch.config_from_dict(d)
     if rope_scaling_override[0]:
         cfg = cfg.with_rope_scaling(rope_scaling_override[1])
+    if hasattr(cfg, "with_tensor_shapes"):
+        # sizes that only the checkpoint knows (config.json does not repeat them)
+        from tokasaurus_amd.weights.loader import tensor_shapes
+
+        cfg = cfg.with_tensor_shapes(tensor_shapes(model_dir))
     return arch, cfg
 
 

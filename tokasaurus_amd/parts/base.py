@@ -24,6 +24,9 @@ import torch
 MATRIX = "matrix"  # a projection or table of floats: engine dtype, N(0, 0.02) when random
 BIAS = "bias"  # a projection's bias vector: engine dtype, N(0, 0.02) when random
 NORM_WEIGHT = "norm_weight"  # a norm's scale vector: 1 + N(0, 0.01) when random
+NORM_OFFSET = "norm_offset"  # a norm's scale stored around zero (the norm multiplies by 1 + w): N(0, 0.01) when random
+VECTOR = "vector"  # a learned vector of another role (a sink, a rate, a step's bias): N(0, 0.5) when random
+CONV = "conv"  # the taps of short convolutions, [channels, taps]: N(0, 0.5) when random
 INT_TABLE = "int_table"  # integer table: kept as int32
 
 
@@ -44,6 +47,11 @@ class CacheNeed:
     num_kv_heads: int
     head_dim: int
     window: int = 0  # 0: every key is kept; > 0: only the last `window` positions are read
+    value_dim: int = 0  # size of a value head where it differs from a key head's (0: the same)
+
+    @property
+    def value_size(self) -> int:
+        return self.value_dim or self.head_dim
 
 
 @dataclass(frozen=True)
@@ -220,6 +228,20 @@ class Mixer(Part):
         rows: torch.Tensor | None,
     ) -> torch.Tensor:
         raise NotImplementedError
+
+    def mix(
+        self,
+        h: torch.Tensor,
+        ctx: StepContext,
+        cache: CacheView | None,
+        state: torch.Tensor | None,
+        rows: torch.Tensor | None,
+        out_f32: bool = False,
+    ) -> torch.Tensor:
+        """The mixer's own output ``mix(h)`` with nothing added (for ``rows`` only when given;
+        ``out_f32``: the last product's 32-bit sums leave unrounded): what a block needs that
+        combines its branches itself.  A mixer need not have it; blocks that call it say so."""
+        raise NotImplementedError(f"{type(self).__name__} gives its output only added to the stream")
 
 
 class FeedForward(Part):

@@ -94,3 +94,93 @@ class PreNormBlock(Block):
         if self.feed_forward.fuses_norm:
             return self.feed_forward.forward(Normed(x, self.ff_norm, prepared), x, emit_norm=next_norm)
         return self.feed_forward.forward(Normed(x, self.ff_norm, prepared).materialize(), x)
+
+
+class NormPair(Part):
+    """The two norms a block with side-by-side branches begins with: both read the same
+    stream, so one pass computes the statistic once and writes both rows."""
+
+    def __init__(self, first, second):
+        self.first, self.second = first, second
+
+    def children(self) -> list[Part]:
+        return [n for n in (self.first, self.second) if n is not None]
+
+    def fused(self) -> bool:
+        return self.second is None or self.first.same_rule(self.second)
+
+    def forward_pair(self, x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor | None]:
+        if not self.fused():
+            return self.first.forward(x), self.second.forward(x)
+        n = self.first
+        _, h1, h2 = ops.residual_norm(x, weights=(n.weight, self.second.weight if self.second is not None else None),
+                                      unit_offset=n.unit_offset, eps=n.eps, out_dtype=n.out_dtype)
+        return h1, h2
+
+
+@BLOCKS.register("parallel_residual")
+class ParallelResidualBlock(Block):
+    """Mixer and feed-forward side by side on a 32-bit residual stream:
+        x <- x + mult * (mixer(norm1(x)) + ff(norm2(x)))
+    both norms of the same x; ``feed_forward`` (and its norm) may be absent.  The stream is
+    32-bit whatever the storage type; the branches hand over their last products' 32-bit sums,
+    and one kernel adds them to the stream and writes the rows of the norms that read the new
+    stream (the next block's pair, or the head's norm).  The norms are ``stream_rmsnorm``s; the
+    mixer must have ``mix`` and the feed-forward ``transform``."""
+
+    fuses_norm = True
+
+    def __init__(self, mixer_norm: PartSpec, mixer: PartSpec, ff_norm: PartSpec | None = None,
+                 feed_forward: PartSpec | None = None, residual_mult: float = 1.0, shared: dict | None = None):
+        shared = shared if shared is not None else {}
+        if (ff_norm is None) != (feed_forward is None):
+            raise ValueError("a feed-forward and its norm come together")
+        self.mixer_norm = build_with_shared(NORMS, mixer_norm, shared)
+        self.mixer = build_with_shared(MIXERS, mixer, shared)
+        self.ff_norm = build_with_shared(NORMS, ff_norm, shared) if ff_norm is not None else None
+        self.feed_forward = build_with_shared(FEED_FORWARDS, feed_forward, shared) if feed_forward is not None else None
+        self.residual_mult = float(residual_mult)
+        self.entry = NormPair(self.mixer_norm, self.ff_norm)
+
+    def children(self) -> list[Part]:
+        return [c for c in (self.mixer_norm, self.mixer, self.ff_norm, self.feed_forward) if c is not None]
+
+    def tensor_specs(self) -> list[TensorSpec]:
+        return [s for c in self.children() for s in c.tensor_specs()]
+
+    def load(self, tensors: dict[str, torch.Tensor], placer: Placer) -> None:
+        for c in self.children():
+            c.load(tensors, placer)
+
+    def entry_norm(self):
+        return self.entry
+
+    def forward(self, x, ctx: StepContext, cache, state, rows, prepared: Prepared | None = None, next_norm=None):
+        if x.dtype != torch.float32:
+            raise TypeError("a parallel_residual block runs on a 32-bit stream (an embedding with stream_f32)")
+        if prepared is not None and prepared.norm is self.entry and prepared.normed is not None:
+            h1, h2 = prepared.normed
+        else:
+            h1, h2 = self.entry.forward_pair(x)
+        a = self.mixer.mix(h1, ctx, cache, state, rows, out_f32=True)
+        if rows is not None:
+            x = ops.gather_rows(x, rows)
+            h2 = ops.gather_rows(h2, rows) if h2 is not None else None
+        b = self.feed_forward.transform(h2, out_f32=True) if self.feed_forward is not None else None
+        # the norms that read the new stream: the next block's pair or a single norm (the head's)
+        first = second = None
+        if isinstance(next_norm, NormPair) and next_norm.fused():
+            first, second = next_norm.first, next_norm.second
+        elif getattr(next_norm, "same_rule", None) is not None:
+            first = next_norm
+        x, g1, g2 = ops.residual_norm(
+            x, (a, b), self.residual_mult,
+            weights=(first.weight if first is not None else None, second.weight if second is not None else None),
+            unit_offset=first.unit_offset if first is not None else False, eps=first.eps if first is not None else 0.0,
+            out_dtype=first.out_dtype if first is not None else torch.float32)
+        tap = ctx.extras.get("stream_tap")
+        if tap is not None:  # a list that collects the stream after every block (tests, debugging)
+            tap.append(x.clone())
+        if first is None:
+            return x
+        return x, Prepared(None, next_norm, (g1, g2) if isinstance(next_norm, NormPair) else g1)

@@ -18,10 +18,16 @@ from tokasaurus_amd.parts.linear import Linear, Placer
 
 @EMBEDDINGS.register("token_embedding")
 class TokenEmbedding(Embedding):
-    def __init__(self, vocab_size: int, hidden_size: int, name: str):
+    def __init__(self, vocab_size: int, hidden_size: int, name: str, scale: float | None = None, stream_f32: bool = False):
+        """``scale``: every row is multiplied by it.  ``stream_f32``: the rows leave in 32-bit
+        whatever the table's storage type (a model that keeps its residual stream in 32-bit)."""
         self.vocab_size = vocab_size
         self.hidden_size = hidden_size
         self.name = name
+        self.scale = None if scale is None else float(scale)
+        self.stream_f32 = bool(stream_f32)
+        if self.scale is not None and not self.stream_f32:
+            raise ValueError("a scaled embedding writes a 32-bit stream (stream_f32=True)")
         self.table: torch.Tensor | None = None
 
     def tensor_specs(self) -> list[TensorSpec]:
@@ -34,14 +40,18 @@ class TokenEmbedding(Embedding):
         )
 
     def forward(self, ctx: StepContext) -> torch.Tensor:
+        if self.stream_f32:
+            return ops.embed_scaled(ctx.token_ids, self.table, 1.0 if self.scale is None else self.scale, ctx.last_token)
         return ops.embed_gather(ctx.token_ids, self.table, ctx.last_token)
 
 
 @HEADS.register("norm_linear")
 class LMHead(Head):
-    def __init__(self, vocab_size: int, hidden_size: int, name: str, norm: PartSpec):
+    def __init__(self, vocab_size: int, hidden_size: int, name: str, norm: PartSpec, softcap: float | None = None):
+        """``softcap``: the logits leave as softcap * tanh(logits / softcap)."""
         self.vocab_size = vocab_size
         self.hidden_size = hidden_size
+        self.softcap = float(softcap) if softcap else None
         self.norm = NORMS.build(norm)
         self.proj = Linear(hidden_size, [name], [vocab_size])
 
@@ -61,4 +71,5 @@ class LMHead(Head):
     takes_out = True
 
     def forward(self, x: torch.Tensor, prepared: Prepared | None = None, out: torch.Tensor | None = None) -> torch.Tensor:
-        return self.proj(Normed(x, self.norm, prepared), out_f32=True, out=out)
+        logits = self.proj(Normed(x, self.norm, prepared), out_f32=True, out=out)
+        return ops.softcap_(logits, self.softcap) if self.softcap is not None else logits

@@ -28,3 +28,8 @@ class SwiGLU(FeedForward):
 
     def forward(self, h: torch.Tensor | Normed, residual: torch.Tensor, emit_norm=None):
         return self.down.with_residual(self.gate_up(h, swiglu=True), residual, emit_norm)
+
+    def transform(self, h: torch.Tensor, out_f32: bool = False) -> torch.Tensor:
+        """The feed-forward's own output, nothing added: for blocks that combine their branches
+        themselves.  ``out_f32``: the down projection's 32-bit sums leave unrounded."""
+        return self.down(self.gate_up(h, swiglu=True), out_f32=out_f32)

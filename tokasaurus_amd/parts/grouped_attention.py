@@ -1,0 +1,140 @@
+"""Grouped-query attention over the paged cache with the pieces that ``paged_attention`` does
+not have, each a parameter: key and value heads of different sizes, a scale of the model's
+choosing, RMS norms of the queries and of the keys over the whole projection (all heads at
+once), a rotation of neighbouring elements of the leading part of a head, a sliding window, a
+learned sink per query head in the softmax's denominator, and keys and values taken from
+another layer's cache (the run entry's ``cache_of``; the mixer then has no key and value
+tensors).
+
+Scores, softmax weights, norms, angles and the rotation are 32-bit arithmetic in either storage
+type.  One kernel norms, rotates and appends (``ops.qk_prepare``); the attention itself is the
+32-bit-arithmetic kernel (``ops.paged_attention_generic``).
+"""
+
+from __future__ import annotations
+
+import torch
+
+from tokasaurus_amd.kernels import ops
+from tokasaurus_amd.parts.base import (
+    MIXERS,
+    NORM_WEIGHT,
+    POSITION_ENCODINGS,
+    VECTOR,
+    CacheNeed,
+    CacheView,
+    Mixer,
+    PartSpec,
+    StepContext,
+    TensorSpec,
+)
+from tokasaurus_amd.parts.linear import Linear, Placer
+from tokasaurus_amd.parts.position import InterleavedRotary
+
+
+@MIXERS.register("grouped_attention")
+class GroupedAttention(Mixer):
+    def __init__(
+        self,
+        hidden_size: int,
+        num_heads: int,
+        num_kv_heads: int,
+        key_dim: int,
+        value_dim: int,
+        scale: float,
+        names: dict[str, str],
+        position: PartSpec | None = None,
+        window: int = 0,
+        cache_window: int | None = None,
+        projection_norm: dict | None = None,
+        sink_name: str | None = None,
+        own_kv: bool = True,
+        shared: dict | None = None,
+    ):
+        """``names``: checkpoint names of the q, k, v, o matrices (k and v only with ``own_kv``).
+        ``projection_norm``: ``{"q": name, "k": name, "eps": eps}``, weights of the whole
+        projections' sizes (k only with ``own_kv``).  ``window``: a query sees itself and the
+        window - 1 positions before it (0: all).  ``cache_window``: how far back the cache keeps
+        keys (0: all): at least ``window``, more when another layer reads this cache further
+        back; by default ``window``.  ``sink_name``: one number a query head."""
+        if num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} query heads are not a multiple of {num_kv_heads} kv heads")
+        self.hidden_size, self.num_heads, self.num_kv_heads = hidden_size, num_heads, num_kv_heads
+        self.key_dim, self.value_dim = int(key_dim), int(value_dim)
+        self.scale = float(scale)
+        self.window = int(window)
+        self.cache_window = self.window if cache_window is None else int(cache_window)
+        if self.cache_window and (not self.window or self.window > self.cache_window):
+            raise ValueError(f"a window of {self.window or 'all'} keys reads further back than the {self.cache_window} the cache keeps")
+        self.own_kv = bool(own_kv)
+        self.projection_norm = dict(projection_norm) if projection_norm else None
+        self.sink_name = sink_name
+        sizes = [num_heads * key_dim] + ([num_kv_heads * key_dim, num_kv_heads * value_dim] if own_kv else [])
+        self.qkv = Linear(hidden_size, [names["q"]] + ([names["k"], names["v"]] if own_kv else []), sizes)
+        self.out = Linear(num_heads * value_dim, [names["o"]], [hidden_size])
+        self.q_norm_weight: torch.Tensor | None = None
+        self.k_norm_weight: torch.Tensor | None = None
+        self.sink: torch.Tensor | None = None
+        self.position = None
+        if position is not None:
+            shared = shared if shared is not None else {}
+            self.position = shared.setdefault(("position", position), POSITION_ENCODINGS.build(position))
+            if not isinstance(self.position, InterleavedRotary) or self.position.dims > key_dim:
+                raise ValueError("grouped_attention rotates neighbouring elements: it takes a rotary_interleaved encoding "
+                                 "of at most a key head's size")
+
+    def tensor_specs(self) -> list[TensorSpec]:
+        specs = self.qkv.tensor_specs() + self.out.tensor_specs()
+        if self.projection_norm:
+            specs.append(TensorSpec(self.projection_norm["q"], (self.num_heads * self.key_dim,), NORM_WEIGHT))
+            if self.own_kv:
+                specs.append(TensorSpec(self.projection_norm["k"], (self.num_kv_heads * self.key_dim,), NORM_WEIGHT))
+        if self.sink_name:
+            specs.append(TensorSpec(self.sink_name, (self.num_heads,), VECTOR))
+        return specs
+
+    def cache_need(self) -> CacheNeed:
+        return CacheNeed(self.num_kv_heads, self.key_dim, self.cache_window,
+                         0 if self.value_dim == self.key_dim else self.value_dim)
+
+    def check_cache(self, page_size: int, dtype: torch.dtype) -> None:
+        ops.check_attention_shape(dtype, self.num_heads, self.num_kv_heads, self.key_dim, page_size,
+                                  value_dim=self.value_dim, generic_only=True)
+
+    def load(self, tensors: dict[str, torch.Tensor], placer: Placer) -> None:
+        self.qkv.load(tensors, placer)
+        self.out.load(tensors, placer)
+
+        def f32(name: str) -> torch.Tensor:
+            return placer.place(("vector_f32", name), lambda: tensors[name].to(torch.float32).contiguous().to(placer.device))
+
+        if self.projection_norm:
+            self.q_norm_weight = f32(self.projection_norm["q"])
+            if self.own_kv:
+                self.k_norm_weight = f32(self.projection_norm["k"])
+        if self.sink_name:
+            self.sink = f32(self.sink_name)
+        if self.position is not None:
+            self.position.prepare(placer.device)
+
+    def _attend(self, h: torch.Tensor, ctx: StepContext, cache: CacheView, rows: torch.Tensor | None) -> torch.Tensor:
+        assert cache is not None, "grouped attention needs a cache"
+        if cache.writable != self.own_kv:
+            raise RuntimeError("a mixer with key and value tensors of its own writes its cache; one without reads another's")
+        nq, nkv, dk, dv = self.num_heads, self.num_kv_heads, self.key_dim, self.value_dim
+        qkv = self.qkv(h)
+        eps = float(self.projection_norm["eps"]) if self.projection_norm else 0.0
+        ops.qk_prepare(qkv, ctx.positions, ctx.token_req, cache.block_table, self.q_norm_weight,
+                       self.k_norm_weight if self.own_kv else None, eps,
+                       self.position.freq if self.position is not None else None,
+                       cache.keys, cache.values, nq, nkv, dk, dv, cache.page_size, write_cache=self.own_kv)
+        attn = ops.paged_attention_generic(qkv, cache.keys, cache.values, cache.block_table, ctx.token_req, ctx.positions,
+                                           nq, nkv, dk, cache.page_size, window=self.window, scale=self.scale,
+                                           value_dim=dv, sink=self.sink)
+        return attn if rows is None else ops.gather_rows(attn, rows)
+
+    def mix(self, h, ctx, cache, state, rows, out_f32: bool = False):
+        return self.out(self._attend(h, ctx, cache, rows), out_f32=out_f32)
+
+    def forward(self, h, residual, ctx, cache, state, rows):
+        return self.out(self._attend(h, ctx, cache, rows), residual=residual)

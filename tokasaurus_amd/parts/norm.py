@@ -6,7 +6,7 @@ from __future__ import annotations
 import torch
 
 from tokasaurus_amd.kernels import ops
-from tokasaurus_amd.parts.base import NORMS, NORM_WEIGHT, Norm, TensorSpec
+from tokasaurus_amd.parts.base import NORMS, NORM_OFFSET, NORM_WEIGHT, Norm, TensorSpec
 from tokasaurus_amd.parts.linear import Placer
 
 
@@ -33,3 +33,38 @@ class RMSNorm(Norm):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return ops.rmsnorm(x, self.weight, self.eps)
+
+
+@NORMS.register("stream_rmsnorm")
+class StreamRMSNorm(Norm):
+    """RMSNorm of a residual stream that is kept in 32-bit whatever the storage type:
+    ``x / sqrt(mean(x^2) + eps) * w`` computed in 32-bit and rounded once to the storage type
+    that the products behind it read.  ``unit_offset``: the checkpoint stores the weight around
+    zero and the norm multiplies by ``1 + w``.  The weight is kept in 32-bit.  A block that
+    updates the stream may write this norm's rows in the same pass (``ops.residual_norm``)."""
+
+    fusable_rms = False  # the few-row product's folded norm has no offset and reads storage-type rows
+
+    def __init__(self, size: int, eps: float, name: str, unit_offset: bool = False):
+        self.size = size
+        self.eps = float(eps)
+        self.name = name
+        self.unit_offset = bool(unit_offset)
+        self.weight: torch.Tensor | None = None
+        self.out_dtype: torch.dtype | None = None
+
+    def tensor_specs(self) -> list[TensorSpec]:
+        return [TensorSpec(self.name, (self.size,), NORM_OFFSET if self.unit_offset else NORM_WEIGHT)]
+
+    def load(self, tensors: dict[str, torch.Tensor], placer: Placer) -> None:
+        host = tensors[self.name]
+        self.weight = placer.place(("vector_f32", self.name), lambda: host.to(dtype=torch.float32).contiguous().to(placer.device))
+        self.out_dtype = placer.dtype
+
+    def same_rule(self, other: "Norm | None") -> bool:
+        """Whether one pass can write this norm's rows and ``other``'s: the same statistic and offset."""
+        return isinstance(other, StreamRMSNorm) and (other.eps, other.unit_offset, other.size) == (self.eps, self.unit_offset, self.size)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return ops.residual_norm(x, weights=(self.weight, None), unit_offset=self.unit_offset, eps=self.eps,
+                                 out_dtype=self.out_dtype)[1]

@@ -64,3 +64,43 @@ class RotaryEncoding(PositionEncoding):
             return
         inv_freq = inverse_frequencies(self.head_dim, self.theta, self.scaling).to(device)
         self.cos, self.sin = ops.rope_table(inv_freq, self.max_positions)
+
+
+def interleaved_frequencies(dims: int, base: float, scaling: dict | None) -> torch.Tensor:
+    """f_i = base^(-2i/dims) for i < dims/2, computed in 64-bit on the host and rounded once to
+    32-bit.  ``scaling`` (``factor``, ``low``, ``high``, ``original``) rescales by wavelength
+    l = 2 pi / f: f stays where l < original/high, becomes f/factor where l > original/low, and
+    between the two is (1 - s) f/factor + s f with s = (original/l - low) / (high - low)."""
+    out = []
+    for i in range(dims // 2):
+        f = float(base) ** (-2.0 * i / dims)
+        if scaling:
+            factor, low, high = float(scaling["factor"]), float(scaling["low"]), float(scaling["high"])
+            original = float(scaling["original"])
+            wavelength = 2.0 * math.pi / f
+            if wavelength > original / low:
+                f = f / factor
+            elif not wavelength < original / high:
+                s = (original / wavelength - low) / (high - low)
+                f = (1.0 - s) * f / factor + s * f
+        out.append(f)
+    return torch.tensor(out, dtype=torch.float64).to(torch.float32)
+
+
+@POSITION_ENCODINGS.register("rotary_interleaved")
+class InterleavedRotary(PositionEncoding):
+    """A rotation of neighbouring elements (2i, 2i+1) of the leading ``dims`` elements of a head
+    by the angle position * f_i.  It keeps the frequencies only: the kernel that rotates
+    multiplies and takes sine and cosine in 32-bit itself, so positions have no upper end."""
+
+    def __init__(self, dims: int, base: float, scaling: dict | None = None):
+        if dims % 2 or dims <= 0:
+            raise ValueError(f"a rotation of pairs needs an even number of elements, got {dims}")
+        self.dims = int(dims)
+        self.base = float(base)
+        self.scaling = dict(scaling) if scaling else None
+        self.freq: torch.Tensor | None = None
+
+    def prepare(self, device: torch.device) -> None:
+        if self.freq is None:
+            self.freq = interleaved_frequencies(self.dims, self.base, self.scaling).to(device)

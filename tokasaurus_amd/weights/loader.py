@@ -69,6 +69,16 @@ def _files_by_tensor(folder: Path) -> dict[str, Path]:
     raise FileNotFoundError(f"no {SINGLE_FILE} or {INDEX_FILE} in {folder}")
 
 
+def tensor_shapes(folder: str | Path) -> dict[str, tuple[int, ...]]:
+    """Name -> shape of every tensor of the checkpoint, from the files' headers (no data is read)."""
+    out: dict[str, tuple[int, ...]] = {}
+    for path in sorted(set(_files_by_tensor(Path(folder)).values())):
+        with safe_open(str(path), framework="pt") as f:
+            for name in f.keys():
+                out[name] = tuple(f.get_slice(name).get_shape())
+    return out
+
+
 def read_tensors(
     folder: str | Path,
     specs: list[TensorSpec],
