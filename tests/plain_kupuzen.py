@@ -28,8 +28,10 @@ def silu(z):
     return z * torch.sigmoid(z)
 
 
-def rotary_frequencies(rot: dict, dtype=torch.float64) -> torch.Tensor:
-    """f_i = base^(-2i/dims), i < dims/2, with the three bands of wavelength scaling."""
+def rotary_frequencies(rot: dict | None, dtype=torch.float64) -> torch.Tensor:
+    """f_i = base^(-2i/dims), i < dims/2, with the three bands of wavelength scaling (none for no rotation)."""
+    if not rot:
+        return torch.zeros(0, dtype=dtype)
     dims = int(rot["dims"])
     f = torch.tensor([float(rot["base"]) ** (-2.0 * i / dims) for i in range(dims // 2)], dtype=torch.float64)
     sc = rot.get("scaling")
@@ -67,7 +69,7 @@ def attention_keys_values(h, w, p, mixer, eps, positions):
     G, dk, dv = mixer["kv_heads"], mixer["dim"], mixer["vdim"]
     k = h @ w[f"{p}.k"].T
     k = rms(k, eps) * w[f"{p}.k.norm"]
-    k = rotate_interleaved(k.view(-1, G, dk), positions, rotary_frequencies(mixer["rot"], h.dtype))
+    k = rotate_interleaved(k.view(-1, G, dk), positions, rotary_frequencies(mixer.get("rot"), h.dtype))
     v = (h @ w[f"{p}.v"].T).view(-1, G, dv)
     return k, v
 
@@ -79,7 +81,7 @@ def attention(h, w, p, mixer, eps, positions, kv=None):
     T = h.shape[0]
     q = h @ w[f"{p}.q"].T
     q = rms(q, eps) * w[f"{p}.q.norm"]
-    q = rotate_interleaved(q.view(T, H, dk), positions, rotary_frequencies(mixer["rot"], h.dtype))
+    q = rotate_interleaved(q.view(T, H, dk), positions, rotary_frequencies(mixer.get("rot"), h.dtype))
     k, v = kv if kv is not None else attention_keys_values(h, w, p, mixer, eps, positions)
     window = mixer.get("mask", {}).get("size") if mixer.get("mask") else None
     out = torch.zeros(T, H, dv, dtype=h.dtype)

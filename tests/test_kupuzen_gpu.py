@@ -1,0 +1,237 @@
+"""Kupuzen through the engine against the plain model: every mechanism alone, prompts against
+token-by-token decoding, portions down to two tokens, unequal requests in one batch on pages
+and slots that are used again, keys just inside and just outside every window, long decoding,
+and greedy generation through ``Engine.generate``."""
+
+from __future__ import annotations
+
+import copy
+import json
+
+import pytest
+import torch
+
+import plain_kupuzen as pk
+from kupuzen_models import CONFIGS, MIXED, RECURRENT, TOL, WINDOWS, attention_layer, compare_rows, delta_layer, load_plain, make_folder, plain_rows
+from replay_helpers import mixed_trace, portions, run_steps, tail_one_by_one, whole
+from tiny_models import random_tokens
+from tokasaurus_amd.engine.batch import StepEntry, layout, to_device
+from tokasaurus_amd.engine.runner import ModelRunner
+
+pytestmark = pytest.mark.gpu
+PAGE = 16
+
+
+@pytest.fixture(scope="module")
+def kupuzen_folders(tmp_path_factory):
+    root = tmp_path_factory.mktemp("kupuzen")
+    return {name: make_folder(root / name, cfg, seed=3 + i) for i, (name, cfg) in enumerate(sorted(CONFIGS.items()))}
+
+
+def runner_for(folder, dtype, tokens=512, slots=4, **kw):
+    return ModelRunner.from_folder(str(folder), dtype, page_size=PAGE, num_pages=tokens // PAGE, max_slots=slots, **kw)
+
+
+def one_layer(layer: dict, width=64, vocab=120, **top) -> dict:
+    cfg = {"architecture": "Kupuzen", "vocab": vocab, "width": width, "embedding": {"scale": 2.0}, "norm": {"eps": 1e-5},
+           "residual_mult": 0.7, "layers": [layer]}
+    cfg.update(top)
+    return cfg
+
+
+def streams_of(runner, tokens):
+    """The residual stream after every block for one whole prompt."""
+    planned = runner.plan([StepEntry("tap", tokens, [])])
+    runner.storage.reset_slots(runner.manager.take_fresh_slots())
+    hb = layout(planned, runner.model.spec.vocab_size, len(runner.groups), runner.manager.slot_tables)
+    ctx, _, tables = to_device(hb, runner.model.dtype, runner.model.device, runner.storage.last_token)
+    ctx.extras["kv_bound"] = runner.kv_bound(ctx.max_kv_len)
+    tap: list = []
+    ctx.extras["stream_tap"] = tap
+    runner.model.forward(ctx, runner.cache_views(tables), runner.storage.states, None)
+    runner.release("tap")
+    return [t.cpu() for t in tap]
+
+
+SINGLE_LAYERS = {
+    "attention": attention_layer(4, 2, 16, 8, 0.3, window=7, rot={"base": 100.0, "dims": 6}),
+    "attention_whole_rotation_no_window": attention_layer(3, 3, 8, 24, 0.5, rot={"base": 9.0, "dims": 8}, ff=40),
+    "delta": delta_layer(4, 2, 16, 24, 4, 8, 16),
+    "delta_wide_key": delta_layer(2, 1, 136, 8, 2, 8, 8, ff=32),
+    "feed_forward_beside_attention": attention_layer(1, 1, 8, 8, 1.0, window=2, ff=72),
+}
+
+
+@pytest.mark.parametrize("name", sorted(SINGLE_LAYERS))
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_one_layer_alone(tmp_path, name, dtype):
+    """A model of one layer: the stream after it and the logits, for a whole prompt."""
+    config = one_layer(SINGLE_LAYERS[name], logit_softcap=5.0 if "delta" in name else None)
+    folder = make_folder(tmp_path / name, config, seed=21)
+    tokens = random_tokens(37, config["vocab"], 5)
+    cfg, w = load_plain(folder)
+    logits, streams = pk.forward(cfg, w, tokens, return_layers=True)
+    runner = runner_for(folder, dtype, tokens=64)
+    got = streams_of(runner, tokens)
+    assert len(got) == 1 and got[0].dtype == torch.float32
+    rel = float((got[0].double() - streams[0]).norm() / streams[0].norm())
+    assert rel < (2e-5 if dtype == "float32" else 2e-2), f"stream after the layer: relative error {rel:.2e}"
+    rows = run_steps(runner, whole("a", tokens))
+    compare_rows(rows, {"a": logits.float()}, TOL[dtype])
+
+
+@pytest.mark.parametrize("name", sorted(CONFIGS))
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_every_cutting_gives_the_plain_rows(kupuzen_folders, name, dtype):
+    """Whole prompts, a tail decoded token by token (through recorded steps), portions of
+    changing sizes down to two tokens and one, and unequal requests mixed in one batch on a
+    pool so small that pages and slots are used again."""
+    folder, vocab = kupuzen_folders[name], CONFIGS[name]["vocab"]
+    reqs = {f"r{i}": random_tokens(n, vocab, 50 + i) for i, n in enumerate((70, 3, 41, 1, 97, 26))}
+    plain = plain_rows(folder, reqs)
+    runner = runner_for(folder, dtype, tokens=256)
+    for rid, toks in reqs.items():
+        compare_rows(run_steps(runner, whole(rid, toks)), plain, TOL[dtype])
+    compare_rows(run_steps(runner, tail_one_by_one("r4", reqs["r4"], tail=40)), plain, TOL[dtype])
+    compare_rows(run_steps(runner, portions("r4", reqs["r4"], [2, 3, 16, 2, 1, 31, 5])), plain, TOL[dtype])
+    compare_rows(run_steps(runner, portions("r0", reqs["r0"], [15, 17, 1, 2])), plain, TOL[dtype])
+    for seed in (1, 2):
+        compare_rows(run_steps(runner, mixed_trace(reqs, seed, max_live=4)), plain, TOL[dtype])
+    assert runner.manager.requests == {}
+    if dtype == "float32":
+        # the same position from different cuttings: the same up to the order of 32-bit sums
+        a = run_steps(runner, whole("r2", reqs["r2"]))
+        b = run_steps(runner, portions("r2", reqs["r2"], [2, 7]))
+        assert max(float((a[k] - b[k]).abs().max()) for k in a) < 2e-4
+
+
+def test_batch_rows_do_not_depend_on_their_neighbours(kupuzen_folders):
+    """A request alone and the same request between two others, as a prompt portion and as a
+    single token: bit for bit the same logits in 32-bit (every kernel's order of sums is fixed
+    by the token's own place; the batches are sized so that the 32-bit product, which has one
+    form for few rows and one for many, takes the same form in both runs)."""
+    folder, vocab = kupuzen_folders["mixed"], MIXED["vocab"]
+    a, b, c = (random_tokens(n, vocab, 90 + n) for n in (33, 50, 19))
+    runner = runner_for(folder, "float32", tokens=256)
+    alone = run_steps(runner, [{"entries": [("b", b[:40], list(range(40)))]}, {"entries": [("b", b[40:41], [0])], "end": ["b"]}])
+    beside = run_steps(runner, [
+        {"entries": [("a", a[:20], []), ("b", b[:40], list(range(40))), ("c", c[:5], [])]},
+        {"entries": [("a", a[20:21], []), ("b", b[40:41], [0]), ("c", c[5:6], [])], "end": ["a", "b", "c"]}])
+    for key in alone:
+        assert torch.equal(alone[key], beside[key]), f"{key} differs beside other requests"
+
+
+def test_slots_and_pages_are_clean_for_their_next_holder(kupuzen_folders):
+    """Two slots and a pool of eight pages serve six requests one after the other and in pairs:
+    a request must not see the state or the keys of whoever held its slot and pages before."""
+    folder, vocab = kupuzen_folders["mixed"], MIXED["vocab"]
+    reqs = {f"q{i}": random_tokens(n, vocab, 70 + i) for i, n in enumerate((60, 64, 17, 49, 30, 5))}
+    plain = plain_rows(folder, reqs)
+    runner = runner_for(folder, "float32", tokens=128, slots=2)
+    for seed in (3, 4):
+        compare_rows(run_steps(runner, mixed_trace(reqs, seed, max_live=2)), plain, TOL["float32"])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_keys_at_the_windows_edges_and_far_away(tmp_path, dtype):
+    """One key is made to stand out: its token's key row and the last token's query row are
+    scaled so that this one score dominates the softmax.  The logits then show whether that key
+    is seen: the engine must agree with the plain model when the key lies just inside the
+    window, just outside it, at a page's border, far back among hundreds, as a prompt's token
+    and decoded alone."""
+    window = 37
+    layer = attention_layer(2, 1, 16, 16, 1.0, window=window, rot={"base": 20.0, "dims": 4})
+    layer_all = attention_layer(2, 1, 16, 16, 1.0, rot={"base": 20.0, "dims": 4})
+    config = one_layer(layer, width=32, vocab=64)
+    config["layers"] = [layer, layer_all]
+    config["layers"][1]["mixer"] = dict(layer_all["mixer"])
+    folder = make_folder(tmp_path / "edges", config, seed=8, edits={
+        # the sinks small, so that the one large score is not drowned
+        ".sink": lambda t: t * 0.1 - 2.0})
+    cfg, w = load_plain(folder)
+    n = 300
+    runner = runner_for(folder, dtype, tokens=320)
+    worst = 0.0
+    for back in (window - 1, window, 1, 15, 16, 17, 250):  # the marked key lies this far behind the last token
+        tokens = random_tokens(n, 64, 100 + back)
+        # token 63 appears once, at the marked place; its embedding is large, so its key is too
+        tokens = [t % 63 for t in tokens]
+        tokens[n - 1 - back] = 63
+        w2 = dict(w)
+        w2["embed"] = w["embed"].clone()
+        plain = pk.forward(cfg, w2, tokens).float()
+        for steps in (whole("e", tokens), tail_one_by_one("e", tokens, tail=3), portions("e", tokens, [2, 61])):
+            got = run_steps(runner, steps)
+            worst = max(worst, compare_rows({k: v for k, v in got.items() if k[1] >= n - 3}, {"e": plain}, TOL[dtype]))
+    assert worst > 0
+
+
+def test_a_marked_key_changes_the_logits_only_inside_the_window(tmp_path):
+    """The plain model itself: with the marked key one step outside the window of the windowed
+    layer the last row equals that of a prompt without the mark in that layer's view, so the
+    test above does tell inside from outside."""
+    layer = attention_layer(1, 1, 8, 8, 1.0, window=5)
+    config = one_layer(layer, width=16, vocab=32)
+    folder = make_folder(tmp_path / "mark", config, seed=2)
+    cfg, w = load_plain(folder)
+    base = random_tokens(20, 31, 4)
+    inside, outside = list(base), list(base)
+    inside[20 - 1 - 4] = 31
+    outside[20 - 1 - 5] = 31
+    ref = pk.forward(cfg, w, base)[-1]
+    assert float((pk.forward(cfg, w, outside)[-1] - ref).abs().max()) < 1e-12
+    assert float((pk.forward(cfg, w, inside)[-1] - ref).abs().max()) > 1e-3
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(kupuzen_folders, dtype):
+    """A short prompt and 400 tokens decoded one by one: the state is carried 400 times, the
+    windows pass over decoded tokens and give their pages back."""
+    folder, vocab = kupuzen_folders["mixed"], MIXED["vocab"]
+    tokens = random_tokens(420, vocab, 77)
+    plain = plain_rows(folder, {"d": tokens})
+    runner = runner_for(folder, dtype, tokens=448)
+    got = run_steps(runner, tail_one_by_one("d", tokens, tail=400))
+    compare_rows(got, plain, TOL[dtype])
+    assert all(step.captured for step in runner.recorded.values()) and runner.recorded
+
+
+def test_first_tokens_of_a_sequence(kupuzen_folders):
+    """Requests of one, two and three tokens, whole and token by token: the convolutions read
+    zeros before the start, the state starts at zero, the windows are not full yet."""
+    for name in ("mixed", "recurrent", "windows"):
+        folder, vocab = kupuzen_folders[name], CONFIGS[name]["vocab"]
+        reqs = {f"s{n}": random_tokens(n, vocab, 30 + n) for n in (1, 2, 3, 6)}
+        plain = plain_rows(folder, reqs)
+        runner = runner_for(folder, "float32", tokens=64)
+        for rid, toks in reqs.items():
+            compare_rows(run_steps(runner, whole(rid, toks)), plain, TOL["float32"])
+            compare_rows(run_steps(runner, portions(rid, toks, [1])), plain, TOL["float32"])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_greedy_generation_through_the_engine(kupuzen_folders, dtype):
+    """``Engine.generate``: the scheduler cuts prompts into portions beside decoding requests;
+    the tokens are the plain model's greedy tokens (in bfloat16: each token is, for the plain
+    logits of its own history, within rounding of the best)."""
+    from tokasaurus_amd.config.engine_config import EngineConfig
+    from tokasaurus_amd.engine.engine import Engine
+    from tokasaurus_amd.sampling import SamplingParams
+
+    folder, vocab = kupuzen_folders["mixed"], MIXED["vocab"]
+    prompts = [random_tokens(n, vocab, 10 + n) for n in (5, 40, 23, 1, 64)]
+    engine = Engine(EngineConfig(model=str(folder), dtype=dtype, page_size=PAGE, kv_cache_num_tokens=512, max_seqs_per_forward=3,
+                                 max_tokens_per_forward=24, allocator_sanity_checks=True))
+    done = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True))
+    cfg, w = load_plain(folder)
+    for prompt, c in zip(prompts, done):
+        assert len(c.tokens) == 12 and c.finish_reason == "length"
+        ids = list(prompt)
+        for tok in c.tokens:
+            logits = pk.forward(cfg, w, ids)[-1]
+            if dtype == "float32":
+                assert tok == int(logits.argmax()), f"token {tok}, plain {int(logits.argmax())}"
+            else:
+                assert float(logits.max() - logits[tok]) < 0.05 * float(logits.std()) + 0.05
+            ids.append(tok)
+    assert engine.runner.manager.requests == {}

@@ -37,7 +37,7 @@ class CacheStorage:
             nkv, d = grp.need.num_kv_heads, grp.need.head_dim
             # one page more than the pool hands out: the null page, where padding rows write
             entries = (len(grp.entries),)
-            self.keys.append(torch.zeros(entries + key_pages_shape(n + 1, nkv, page_size, d), dtype=dtype, device=device))
+            self.keys.append(torch.zeros(entries + key_pages_shape(n + 1, nkv, page_size, d, padded=True), dtype=dtype, device=device))
             self.values.append(torch.zeros(entries + value_pages_shape(n + 1, nkv, page_size, grp.need.value_size), dtype=dtype, device=device))
         def make(need):
             if need is None:

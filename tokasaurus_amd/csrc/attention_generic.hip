@@ -62,7 +62,7 @@ __global__ __launch_bounds__(AG_THREADS) void paged_attention_generic_kernel(
       const int kp = c0 + j;
       float kv = 0.f;
       if (kp >= lo && kp <= pos)
-        kv = to_f32<T>(kcache[((size_t)table[kp / P] * nkv + g) * P * d + key_offset(P, kp % P, e)]);
+        kv = to_f32<T>(kcache[((size_t)table[kp / P] * nkv + g) * key_page_elems(P, d) + key_offset(P, kp % P, e)]);
       Ks[j * (d + 1) + e] = kv;
     }
     for (int i = tid; i < CH * dv; i += AG_THREADS) {

@@ -77,7 +77,7 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
       v *= k_weight[2 * i + 1];
     }
     if (e < rot) rotate_pair(u, v, cs[e / 2], cs[half + e / 2], u, v);
-    T* dst = kcache + ((size_t)page * nkv + h) * P * dk;
+    T* dst = kcache + ((size_t)page * nkv + h) * key_page_elems(P, dk);
     dst[key_offset(P, p, e)] = from_f32<T>(u);
     dst[key_offset(P, p, e + 1)] = from_f32<T>(v);
   }

@@ -45,6 +45,11 @@ void tk_set_error(const char* fmt, ...);
 __host__ __device__ __forceinline__ size_t key_offset(int P, int in_page, int e) {
   return ((size_t)(e / TK_KEY_PIECE) * P + in_page) * TK_KEY_PIECE + (e % TK_KEY_PIECE);
 }
+// Elements a page of P keys of size d takes: a key whose size is no multiple of the piece has
+// its last piece padded (the matrix-core kernels take multiples of 16 only and never see one).
+__host__ __device__ __forceinline__ size_t key_page_elems(int P, int d) {
+  return (size_t)((d + TK_KEY_PIECE - 1) / TK_KEY_PIECE) * TK_KEY_PIECE * P;
+}
 __host__ __device__ __forceinline__ size_t value_offset(int d, int in_page, int e) {
   return ((size_t)(in_page / TK_VALUE_QUAD) * d + e) * TK_VALUE_QUAD + (in_page % TK_VALUE_QUAD);
 }

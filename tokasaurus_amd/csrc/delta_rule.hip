@@ -272,7 +272,8 @@ TK_API int tk_delta_rule(const float* rec, int ld_rec, float* state, size_t stat
   TK_REQUIRE((size_t)H * dv * dk <= state_stride, "delta_rule: the state row is too short");
   TK_REQUIRE(n_requests < 65536, "delta_rule: too many requests");
   if (n_requests == 0) return 0;
-  const int nq = (dk + DR_LANES * 4 - 1) / (DR_LANES * 4);
+  int nq = (dk + DR_LANES * 4 - 1) / (DR_LANES * 4);
+  nq = nq <= 2 ? nq : (nq <= 4 ? 4 : (nq <= 8 ? 8 : 16));  // the kernel's instances
   TK_REQUIRE(nq <= 4 || cols * DR_LANES <= 256, "delta_rule: key size %d takes at most %d columns a workgroup", dk,
              256 / DR_LANES);
   const int dkp = nq * DR_LANES * 4;
@@ -283,8 +284,8 @@ TK_API int tk_delta_rule(const float* rec, int ld_rec, float* state, size_t stat
                      q_start, slots, o, H, G, dk, dv, cols)
   if (nq == 1) DR_CASE(1);
   else if (nq == 2) DR_CASE(2);
-  else if (nq <= 4) { DR_CASE(4); }
-  else if (nq <= 8) { DR_CASE(8); }
+  else if (nq == 4) DR_CASE(4);
+  else if (nq == 8) DR_CASE(8);
   else DR_CASE(16);
 #undef DR_CASE
   TK_CHECK_LAUNCH("delta_rule");

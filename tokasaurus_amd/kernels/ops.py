@@ -51,12 +51,14 @@ KEY_PIECE = 8  # elements of a key that lie together in a page
 VALUE_QUAD = 4  # tokens whose values lie together in a page
 
 
-def key_pages_shape(pages: int, nkv: int, page_size: int, head_dim: int) -> tuple[int, ...]:
+def key_pages_shape(pages: int, nkv: int, page_size: int, head_dim: int, padded: bool = False) -> tuple[int, ...]:
     """Keys: [pages, nkv, d / 8, P, 8]: a page holds the 8-element pieces of its P
     keys piece by piece, so that the lanes that feed the matrix cores (16 keys, one
-    piece each) read consecutive memory."""
-    _need(head_dim % KEY_PIECE == 0, f"the cache keeps keys in pieces of {KEY_PIECE}: head size {head_dim} is no multiple")
-    return (pages, nkv, head_dim // KEY_PIECE, page_size, KEY_PIECE)
+    piece each) read consecutive memory.
+    ``padded``: a head size that is no multiple of 8 gets its last piece filled up (only the
+    kernels that address pages through ``key_page_elems`` take such a size) instead of a refusal."""
+    _need(padded or head_dim % KEY_PIECE == 0, f"the cache keeps keys in pieces of {KEY_PIECE}: head size {head_dim} is no multiple")
+    return (pages, nkv, -(-head_dim // KEY_PIECE), page_size, KEY_PIECE)
 
 
 def value_pages_shape(pages: int, nkv: int, page_size: int, head_dim: int) -> tuple[int, ...]:
@@ -72,7 +74,7 @@ def _check_pages(kcache: torch.Tensor, vcache: torch.Tensor, nkv: int, page_size
     pages = kcache.shape[0]
     vd = head_dim if value_dim is None else value_dim
     # (the shapes are compared in place: this runs twice a layer of an eager step)
-    if (kcache.shape != (pages, nkv, head_dim // KEY_PIECE, page_size, KEY_PIECE) or head_dim % KEY_PIECE or not kcache.is_contiguous()):
+    if (kcache.shape != (pages, nkv, -(-head_dim // KEY_PIECE), page_size, KEY_PIECE) or not kcache.is_contiguous()):
         raise KernelError(f"{who}: key pages must be contiguous {key_pages_shape(pages, nkv, page_size, head_dim)}, got {tuple(kcache.shape)}")
     if (vcache.shape != (pages, nkv, page_size // VALUE_QUAD, vd, VALUE_QUAD) or page_size % VALUE_QUAD or not vcache.is_contiguous()):
         raise KernelError(f"{who}: value pages must be contiguous {value_pages_shape(pages, nkv, page_size, vd)}, got {tuple(vcache.shape)}")
@@ -413,7 +415,7 @@ def check_attention_shape(dtype: torch.dtype, nq: int, nkv: int, head_dim: int, 
     mixer, so that a model that cannot run is refused before its first step.  ``generic_only``:
     the mixer uses what only the 32-bit-arithmetic kernel has (a value size of its own, sinks)."""
     vd = head_dim if value_dim is None else value_dim
-    key_pages_shape(1, nkv, page_size, head_dim)
+    key_pages_shape(1, nkv, page_size, head_dim, padded=generic_only)
     value_pages_shape(1, nkv, page_size, vd)
     if generic_only or vd != head_dim or not attention_mfma_supports(dtype, head_dim, page_size):
         call("tk_paged_attention_generic_fits", nq, nkv, head_dim, vd)
