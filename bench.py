@@ -82,6 +82,12 @@ def parse() -> argparse.Namespace:
                    help="instead of the decode steps, a case that shapes of one length do not show (prints its own line): "
                         "chunked-prefill: one prompt of --context tokens in portions of --portion tokens; "
                         "mixed-decode: decode steps of --batch - 1 requests of --short tokens beside one of --context tokens")
+    p.add_argument("--design", default=None, choices=["kupuzen"],
+                   help="instead of the decode steps: prefill and decode of this design at layer sizes of --design-sizes "
+                        "beside the Llama shape of equal width, heads, feed-forward and layers (prints its own line)")
+    p.add_argument("--design-sizes", default="1b,3b", help="which sizes of DESIGN_SIZES, comma separated")
+    p.add_argument("--design-layers", type=int, default=8, help="layers of both models in the --design comparison")
+    p.add_argument("--design-context", type=int, default=4096, help="context at which the --design decode steps end")
     p.add_argument("--portion", type=int, default=128)
     p.add_argument("--short", type=int, default=2048)
     return p.parse_args()
@@ -327,6 +333,67 @@ def time_prefill(runner, n: int, reps: int = 10) -> tuple[float, dict]:
     return sum(times) / len(times) / 1e3, summary(times)
 
 
+# Layer sizes for the --design comparison: a Llama shape and a Kupuzen of the same width, feed-forward, layers and
+# vocabulary; its attention layers have the Llama heads (a window of 1,024 keys, sinks, whole-projection norms), its
+# delta-rule layers half as many heads of twice the size, three of them to every attention layer.
+DESIGN_SIZES = {
+    "1b": dict(llama=LLAMA_1B, delta_heads=16, delta_dim=128, window=1024, rank=64),
+    "3b": dict(llama=LLAMA_3B, delta_heads=12, delta_dim=128, window=1024, rank=96),
+    "8b": dict(llama=LLAMA_8B, delta_heads=16, delta_dim=128, window=1024, rank=128),
+}
+
+
+def kupuzen_like(size: dict, layers: int) -> dict:
+    ll = size["llama"]
+    d = ll["hidden_size"] // ll["num_attention_heads"]
+    ff = {"kind": "dense", "ff": ll["intermediate_size"]}
+    attention = {"type": "attention", "mlp": ff, "mixer": {
+        "heads": ll["num_attention_heads"], "kv_heads": ll["num_key_value_heads"], "dim": d, "vdim": d, "scale": d ** -0.5,
+        "mask": {"size": size["window"]},
+        "rot": {"base": ll["rope_theta"], "dims": d, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}}
+    delta = {"type": "channel_delta", "mlp": ff, "mixer": {
+        "heads": size["delta_heads"], "kv_heads": size["delta_heads"], "dim": size["delta_dim"], "vdim": size["delta_dim"],
+        "conv": 4, "decay_rank": size["rank"], "gate_rank": size["rank"]}}
+    return {"architecture": "Kupuzen", "vocab": ll["vocab_size"], "width": ll["hidden_size"], "embedding": {"scale": 1.0},
+            "norm": {"eps": 1e-6}, "residual_mult": 1.0, "logit_softcap": 30.0,
+            "layers": [attention if i % 4 == 3 else delta for i in range(layers)]}
+
+
+def run_design(args) -> int:
+    """Prefill of one prompt and decode steps of the new design beside the Llama shape of equal
+    size, both with seeded random weights through the same runner and engine."""
+    import torch
+
+    out = {"metric": f"prefill and decode of {args.design} beside the Llama shape of equal size", "unit": "tokens/s",
+           "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "layers": args.design_layers, "sizes": {}}
+    batches = [int(b) for b in args.points.split(",") if b] or [1]
+    ctx = args.design_context
+    for name in [x for x in args.design_sizes.split(",") if x]:
+        size = DESIGN_SIZES[name]
+        configs = {"llama": dict(size["llama"], num_hidden_layers=args.design_layers),
+                   args.design: kupuzen_like(size, args.design_layers)}
+        rec = {}
+        for model, cfgd in configs.items():
+            runner = build_runner(cfgd, args.dtype, max(batches) * ctx, max(batches), ctx, use_graphs=not args.eager)
+            one = {}
+            for n in (512, args.prefill_tokens):
+                pdt, _ = time_prefill(runner, n, reps=5)
+                one[f"prefill_{n}_tok_per_s"] = round(n / pdt, 1)
+                one[f"prefill_{n}_ms"] = round(pdt * 1e3, 3)
+            for b in batches:
+                dt, _, stats = time_decode(runner, args, b, ctx, min(args.steps, 32), min(args.warmup, 4))
+                one[f"decode_b{b}_tok_per_s"] = round(b / dt, 1)
+                one[f"decode_b{b}_ms"] = stats["mean"]
+            rec[model] = one
+            say(f"{name} {model}: {one}")
+            del runner
+            torch.cuda.empty_cache()
+        rec["ratio"] = {k: round(rec[args.design][k] / rec["llama"][k], 3) for k in rec["llama"] if k.endswith("tok_per_s")}
+        out["sizes"][name] = rec
+    print(json.dumps(out))
+    return 0
+
+
 def run_scenario(args) -> int:
     """Cases that requests of one length do not show: a long prompt in short portions (each walks
     the whole past), and one long request decoding among short ones."""
@@ -388,6 +455,8 @@ def main() -> int:
         return run_workload(args)
     if args.scenario is not None:
         return run_scenario(args)
+    if args.design is not None:
+        return run_design(args)
     model_name, shape = SHAPES[args.shape]
     cfgd = dict(shape)
     model_layers = cfgd["num_hidden_layers"]
