@@ -56,6 +56,8 @@ def streams_of(runner, tokens):
 SINGLE_LAYERS = {
     "attention": attention_layer(4, 2, 16, 8, 0.3, window=7, rot={"base": 100.0, "dims": 6}),
     "attention_whole_rotation_no_window": attention_layer(3, 3, 8, 24, 0.5, rot={"base": 9.0, "dims": 8}, ff=40),
+    "attention_matrix_core_sizes": attention_layer(8, 2, 40, 32, 0.3, window=19, rot={"base": 100.0, "dims": 10}),
+    "attention_matrix_core_sizes_odd_group": attention_layer(6, 2, 8, 16, 0.3, rot={"base": 100.0, "dims": 8}),
     "delta": delta_layer(4, 2, 16, 24, 4, 8, 16),
     "delta_wide_key": delta_layer(2, 1, 136, 8, 2, 8, 8, ff=32),
     "feed_forward_beside_attention": attention_layer(1, 1, 8, 8, 1.0, window=2, ff=72),

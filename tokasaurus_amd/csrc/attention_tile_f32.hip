@@ -1,0 +1,211 @@
+// Paged attention in 32-bit arithmetic on the matrix cores (v_mfma_f32_16x16x4_f32): scores,
+// softmax weights and the weighted values are 32-bit products of 32-bit operands, whatever the
+// storage type of queries, keys and values.  For mixers that ask for exactly that: a sliding
+// window, key and value heads of different sizes, a scale of the model's choosing and a
+// learned sink per query head in the softmax's denominator.
+//
+// A wavefront owns a tile of 16 "columns": tt = 16 / gg neighbouring tokens of one request
+// times gg neighbouring query heads of one kv head (gg = 1 for prompt portions; up to 16 for
+// single decoded tokens, so that the heads that share keys share their loads).  It walks the
+// keys in steps of 16, at absolute multiples of 16, from the first step that its earliest
+// column sees to the last that its latest column sees:
+//   S^T = K Q^T       keys as the first operand: a lane then holds, for its column (lane % 16),
+//                     the scores of keys 4 * (lane / 16) + i, i < 4
+//   O^T += V^T P^T    which is exactly its second operand here (the order of the sum over the
+//                     16 keys is a free choice: slot lane / 16 of product i is key 4 * (lane / 16) + i)
+// The sum over a head's elements is permuted the same way: a lane loads whole 8-element pieces
+// of its key (the page layout's unit) and of its query, piece lane / 16 + 4 m.
+//   K pages: [page][kv head][dk / 8][P][8]    V pages: [page][kv head][P / 4][dv][4]
+// Needs dk % 8 == 0, dv % 16 == 0, P % 16 == 0 (a step of 16 keys lies inside one page).
+#include "common.h"
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+#define AT_WAVES 4
+#define AT_MAX_KM 8   // dk <= 256
+#define AT_MAX_VT 16  // dv <= 256
+
+template <typename T, int KM, int VT>
+__global__ __launch_bounds__(AT_WAVES * TK_WAVE) void attention_tile_f32_kernel(
+    const T* __restrict__ q, int q_stride, T* __restrict__ out, int out_stride, const T* __restrict__ kcache,
+    const T* __restrict__ vcache, const int* __restrict__ block_table, int table_stride,
+    const int* __restrict__ q_start, const int* __restrict__ kv_len, const int* __restrict__ tile_req,
+    const int* __restrict__ tile_row0, int nq, int nkv, int dk, int dv, int P, int window, float scale,
+    const float* __restrict__ sink, int gg) {
+  const int lane = threadIdx.x & (TK_WAVE - 1), wave = threadIdx.x / TK_WAVE;
+  const int group = nq / nkv;
+  const int blocks_per_kv = group / gg;  // head blocks of gg heads
+  const int hb = blockIdx.y * AT_WAVES + wave;
+  if (hb >= nkv * blocks_per_kv) return;
+  const int kvh = hb / blocks_per_kv;
+  const int head0 = kvh * group + (hb % blocks_per_kv) * gg;
+  const int tile = blockIdx.x;
+  const int r = tile_req[tile];
+  const int row0 = tile_row0[tile];
+  const int tt = 16 / gg;
+  const int col = lane & 15, c = lane >> 4;
+  // this lane's column: a token and a query head
+  const int tok = row0 + col / gg;
+  const int head = head0 + col % gg;
+  const int q_end = q_start[r + 1];
+  const int kv = kv_len[r];
+  const bool live = tok < q_end;
+  const int n_tok = min(tt, q_end - row0);
+  const int pos0 = kv - (q_end - row0);         // position of the tile's first token
+  const int pos = pos0 + col / gg;              // of this column's token
+  const int last = pos0 + n_tok - 1;
+  const int lo_tile = window > 0 ? max(0, pos0 - window + 1) : 0;
+  const int* table = block_table + (size_t)r * table_stride;
+  const int pieces = dk / 8;
+
+  // the column's query, piece c + 4 m
+  float qv[KM][8];
+#pragma unroll
+  for (int m = 0; m < KM; ++m) {
+    const int piece = c + 4 * m;
+    const bool in = live && piece < pieces;
+    const T* src = q + (size_t)(in ? tok : 0) * q_stride + (size_t)head * dk + (in ? piece : 0) * 8;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) qv[m][e] = in ? to_f32<T>(src[e]) : 0.f;
+  }
+
+  v4f o[VT];
+#pragma unroll
+  for (int t = 0; t < VT; ++t) o[t] = (v4f){0.f, 0.f, 0.f, 0.f};
+  float m_run = -INFINITY, l_run = 0.f;  // l_run: this lane's share of the column's sum
+
+  for (int k0 = (lo_tile / 16) * 16; k0 <= last; k0 += 16) {
+    const int page = max(table[k0 / P], 0);
+    const int in_page = k0 % P;
+    // S^T = K Q^T: this lane feeds key k0 + col, pieces c + 4 m
+    const T* kbase = kcache + ((size_t)page * nkv + kvh) * key_page_elems(P, dk);
+    v4f s = (v4f){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int m = 0; m < KM; ++m) {
+      const int piece = c + 4 * m;
+      float kk[8];
+      const T* src = kbase + key_offset(P, in_page + col, (piece < pieces ? piece : 0) * 8);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) kk[e] = piece < pieces ? to_f32<T>(src[e]) : 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) s = __builtin_amdgcn_mfma_f32_16x16x4f32(kk[e], qv[m][e], s, 0, 0, 0);
+    }
+    // this lane now holds, for its column, keys k0 + 4 c + i
+    float sc[4];
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int kp = k0 + 4 * c + i;
+      const bool seen = live && kp <= pos && (window <= 0 || pos - kp < window);
+      sc[i] = seen ? s[i] * scale : -INFINITY;
+      tmax = fmaxf(tmax, sc[i]);
+    }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, TK_WAVE));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, TK_WAVE));
+    const float m_new = fmaxf(m_run, tmax);
+    float p[4];
+    float alpha = 1.f;
+    if (m_new == -INFINITY) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) p[i] = 0.f;
+    } else {
+      alpha = (m_run == -INFINITY) ? 0.f : expf(m_run - m_new);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) p[i] = (sc[i] == -INFINITY) ? 0.f : expf(sc[i] - m_new);
+    }
+    m_run = m_new;
+    l_run = l_run * alpha + ((p[0] + p[1]) + (p[2] + p[3]));
+    // O^T += V^T P^T: this lane feeds value element 16 t + col of keys k0 + 4 c + i
+    const T* vbase = vcache + ((size_t)page * nkv + kvh) * P * dv;
+#pragma unroll
+    for (int t = 0; t < VT; ++t) {
+      if (16 * t < dv) {
+        const T* src = vbase + value_offset(dv, in_page + 4 * c, 16 * t + col);
+        float vv[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) vv[i] = to_f32<T>(src[i]);
+        v4f acc = o[t] * alpha;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(vv[i], p[i], acc, 0, 0, 0);
+        o[t] = acc;
+      }
+    }
+  }
+  // the column's sum, from the four lanes that share it (always in this order)
+  float l = l_run;
+  l += __shfl_xor(l, 16, TK_WAVE);
+  l += __shfl_xor(l, 32, TK_WAVE);
+  float keep = 1.f;
+  if (sink && live) {
+    // the sink joins the softmax like one more score: the maximum may rise to it
+    const float sk = sink[head], m_all = fmaxf(m_run, sk);
+    keep = (m_run == -INFINITY) ? 0.f : expf(m_run - m_all);
+    l = l * keep + expf(sk - m_all);
+  }
+  if (!live) return;
+  const float inv = keep / l;
+  T* dst = out + (size_t)tok * out_stride + (size_t)head * dv;
+#pragma unroll
+  for (int t = 0; t < VT; ++t) {
+    if (16 * t < dv) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) dst[16 * t + 4 * c + i] = from_f32<T>(o[t][i] * inv);
+    }
+  }
+}
+
+// Whether this kernel takes the shape (else the caller uses the plain 32-bit kernel).
+TK_API int tk_attention_tile_f32_fits(int nq, int nkv, int dk, int dv, int P) {
+  return (nq > 0 && nkv > 0 && nq % nkv == 0 && dk > 0 && dk % 8 == 0 && dk <= 32 * AT_MAX_KM && dv > 0 && dv % 16 == 0 &&
+          dv <= 16 * AT_MAX_VT && P > 0 && P % 16 == 0) ? 1 : 0;
+}
+
+template <typename T, int KM, int VT>
+static void at_launch(dim3 grid, hipStream_t stream, const void* q, int q_stride, void* out, int out_stride,
+                      const void* kcache, const void* vcache, const int* block_table, int table_stride,
+                      const int* q_start, const int* kv_len, const int* tile_req, const int* tile_row0, int nq,
+                      int nkv, int dk, int dv, int P, int window, float scale, const float* sink, int gg) {
+  hipLaunchKernelGGL((attention_tile_f32_kernel<T, KM, VT>), grid, dim3(AT_WAVES * TK_WAVE), 0, stream, (const T*)q,
+                     q_stride, (T*)out, out_stride, (const T*)kcache, (const T*)vcache, block_table, table_stride,
+                     q_start, kv_len, tile_req, tile_row0, nq, nkv, dk, dv, P, window, scale, sink, gg);
+}
+
+TK_API int tk_attention_tile_f32(int dt, const void* q, int q_stride, void* out, int out_stride, const void* kcache,
+                                 const void* vcache, const int* block_table, int table_stride, const int* q_start,
+                                 const int* kv_len, const int* tile_req, const int* tile_row0, int n_tiles, int nq,
+                                 int nkv, int dk, int dv, int P, int window, float scale, const float* sink, int gg,
+                                 hipStream_t stream) {
+  TK_REQUIRE(tk_attention_tile_f32_fits(nq, nkv, dk, dv, P), "attention_tile_f32: shape nq=%d nkv=%d dk=%d dv=%d P=%d not taken",
+             nq, nkv, dk, dv, P);
+  const int group = nq / nkv;
+  TK_REQUIRE(gg >= 1 && gg <= 16 && (gg & (gg - 1)) == 0 && group % gg == 0, "attention_tile_f32: %d heads a tile of a group of %d", gg, group);
+  TK_REQUIRE(q_stride >= nq * dk && out_stride >= nq * dv, "attention_tile_f32: row strides too short");
+  if (n_tiles <= 0) return 0;
+  const int head_blocks = nkv * (group / gg);
+  const dim3 grid(n_tiles, (head_blocks + AT_WAVES - 1) / AT_WAVES);
+  TK_REQUIRE(grid.y < 65536, "attention_tile_f32: too many heads");
+  const int km = (dk + 31) / 32, vt = dv / 16;
+#define AT_ARGS grid, stream, q, q_stride, out, out_stride, kcache, vcache, block_table, table_stride, q_start, kv_len, \
+                tile_req, tile_row0, nq, nkv, dk, dv, P, window, scale, sink, gg
+#define AT_VT(T, KMV)                                      \
+  do {                                                     \
+    if (vt <= 2) at_launch<T, KMV, 2>(AT_ARGS);            \
+    else if (vt <= 4) at_launch<T, KMV, 4>(AT_ARGS);       \
+    else if (vt <= 8) at_launch<T, KMV, 8>(AT_ARGS);       \
+    else at_launch<T, KMV, 16>(AT_ARGS);                   \
+  } while (0)
+#define AT_KM(T)                       \
+  do {                                 \
+    if (km <= 1) AT_VT(T, 1);          \
+    else if (km <= 2) AT_VT(T, 2);     \
+    else if (km <= 4) AT_VT(T, 4);     \
+    else AT_VT(T, 8);                  \
+  } while (0)
+  if (dt == TK_F32) AT_KM(float);
+  else AT_KM(bf16_t);
+#undef AT_KM
+#undef AT_VT
+#undef AT_ARGS
+  TK_CHECK_LAUNCH("attention_tile_f32");
+  return 0;
+}

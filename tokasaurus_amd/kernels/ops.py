@@ -1202,6 +1202,52 @@ def qk_prepare(
          n, nq, nkv if write_cache else 0, key_dim, value_dim, rot, page_size, 1 if write_cache else 0, _stream())
 
 
+def attention_tile_f32_fits(nq: int, nkv: int, key_dim: int, value_dim: int, page_size: int) -> bool:
+    """Whether the 32-bit matrix-core attention takes the shape (key size a multiple of 8 up to
+    256, value size a multiple of 16 up to 256, pages of a multiple of 16 keys)."""
+    return bool(load("core").tk_attention_tile_f32_fits(nq, nkv, key_dim, value_dim, page_size))
+
+
+def attention_tile_heads(group: int, max_q_len: int) -> int:
+    """Query heads of one kv head that share a tile of 16 columns: one for prompt portions (16
+    tokens a tile), as many as the group has (the largest power of two that divides it, at most
+    16) when every request brings one token."""
+    if max_q_len > 1:
+        return 1
+    gg = 1
+    while gg < 16 and group % (gg * 2) == 0:
+        gg *= 2
+    return gg
+
+
+def attention_tile_f32(
+    q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, block_table: torch.Tensor, q_start: torch.Tensor,
+    kv_len: torch.Tensor, tile_req: torch.Tensor, tile_row0: torch.Tensor, nq: int, nkv: int, key_dim: int,
+    value_dim: int, page_size: int, heads_a_tile: int, window: int = 0, scale: float = 1.0,
+    sink: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """Attention in 32-bit arithmetic on the matrix cores: every token of the step over its
+    request's pages; ``tile_req`` / ``tile_row0`` name each tile's request and its first token's
+    row (a tile holds 16 / heads_a_tile neighbouring tokens of one request).  Window, scale,
+    value size and sinks as in ``paged_attention_generic``; returns [tokens, nq * value_dim]."""
+    _gpu(q, kcache, vcache, block_table, q_start, kv_len, tile_req, tile_row0, sink)
+    _need(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= nq * key_dim,
+          "attention: q must be 2-d with unit inner stride and nq*d leading columns")
+    for t, name in ((block_table, "block_table"), (q_start, "q_start"), (kv_len, "kv_len"), (tile_req, "tile_req"), (tile_row0, "tile_row0")):
+        _i32(t, name)
+    _need(block_table.dim() == 2 and tile_req.numel() == tile_row0.numel() and q_start.numel() == kv_len.numel() + 1,
+          "attention: block_table [requests, width], one request and one row a tile, one length a request")
+    _need(sink is None or (sink.shape == (nq,) and sink.dtype == torch.float32 and sink.is_contiguous()),
+          f"attention: the sinks must be contiguous float32 [{nq}]")
+    _check_pages(kcache, vcache, nkv, page_size, key_dim, q.dtype, "attention", value_dim)
+    out = torch.empty((q.shape[0], nq * value_dim), dtype=q.dtype, device=q.device)
+    call("tk_attention_tile_f32", dtype_code(q.dtype), q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0),
+         kcache.data_ptr(), vcache.data_ptr(), block_table.data_ptr(), block_table.stride(0), q_start.data_ptr(),
+         kv_len.data_ptr(), tile_req.data_ptr(), tile_row0.data_ptr(), tile_req.numel(), nq, nkv, key_dim, value_dim,
+         page_size, int(window), float(scale), sink.data_ptr() if sink is not None else None, int(heads_a_tile), _stream())
+    return out
+
+
 # --------------------------------------------------------------------------
 # the gated delta rule with a decay per key channel
 # --------------------------------------------------------------------------

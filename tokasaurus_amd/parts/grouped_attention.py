@@ -7,8 +7,10 @@ another layer's cache (the run entry's ``cache_of``; the mixer then has no key a
 tensors).
 
 Scores, softmax weights, norms, angles and the rotation are 32-bit arithmetic in either storage
-type.  One kernel norms, rotates and appends (``ops.qk_prepare``); the attention itself is the
-32-bit-arithmetic kernel (``ops.paged_attention_generic``).
+type.  One kernel norms, rotates and appends (``ops.qk_prepare``); the attention itself runs on
+the matrix cores' 32-bit products (``ops.attention_tile_f32``: tiles of 16 tokens for prompt
+portions, of the heads that share a kv head for single tokens) or, for sizes that kernel does
+not take, on the plain 32-bit kernel (``ops.paged_attention_generic``).
 """
 
 from __future__ import annotations
@@ -16,6 +18,7 @@ from __future__ import annotations
 import torch
 
 from tokasaurus_amd.kernels import ops
+from tokasaurus_amd.kernels.upload import upload
 from tokasaurus_amd.parts.base import (
     MIXERS,
     NORM_WEIGHT,
@@ -30,6 +33,24 @@ from tokasaurus_amd.parts.base import (
 )
 from tokasaurus_amd.parts.linear import Linear, Placer
 from tokasaurus_amd.parts.position import InterleavedRotary
+
+
+def tile_plan(ctx: StepContext, tokens_a_tile: int) -> tuple[torch.Tensor, torch.Tensor]:
+    """The step's rows cut into tiles of up to ``tokens_a_tile`` neighbouring tokens of one
+    request: for every tile its request and its first row.  Made once a step and shared by
+    the layers; a step that is recorded keeps it for its replays."""
+    key = ("tile_plan", tokens_a_tile)
+    plan = ctx.extras.get(key)
+    if plan is None:
+        req, row0 = [], []
+        for r in range(ctx.num_requests):
+            a, b = ctx.host_q_start[r], ctx.host_q_start[r + 1]
+            for first in range(a, b, tokens_a_tile):
+                req.append(r)
+                row0.append(first)
+        dev = upload(req + row0, torch.int32, ctx.device)
+        plan = ctx.extras[key] = (dev[: len(req)], dev[len(req):])
+    return plan
 
 
 @MIXERS.register("grouped_attention")
@@ -128,9 +149,16 @@ class GroupedAttention(Mixer):
                        self.k_norm_weight if self.own_kv else None, eps,
                        self.position.freq if self.position is not None else None,
                        cache.keys, cache.values, nq, nkv, dk, dv, cache.page_size, write_cache=self.own_kv)
-        attn = ops.paged_attention_generic(qkv, cache.keys, cache.values, cache.block_table, ctx.token_req, ctx.positions,
-                                           nq, nkv, dk, cache.page_size, window=self.window, scale=self.scale,
-                                           value_dim=dv, sink=self.sink)
+        if ops.attention_tile_f32_fits(nq, nkv, dk, dv, cache.page_size):
+            gg = ops.attention_tile_heads(nq // nkv, ctx.max_q_len)
+            tile_req, tile_row0 = tile_plan(ctx, 16 // gg)
+            attn = ops.attention_tile_f32(qkv, cache.keys, cache.values, cache.block_table, ctx.q_start, ctx.kv_len,
+                                          tile_req, tile_row0, nq, nkv, dk, dv, cache.page_size, gg,
+                                          window=self.window, scale=self.scale, sink=self.sink)
+        else:  # sizes that the matrix-core kernel does not take
+            attn = ops.paged_attention_generic(qkv, cache.keys, cache.values, cache.block_table, ctx.token_req, ctx.positions,
+                                               nq, nkv, dk, cache.page_size, window=self.window, scale=self.scale,
+                                               value_dim=dv, sink=self.sink)
         return attn if rows is None else ops.gather_rows(attn, rows)
 
     def mix(self, h, ctx, cache, state, rows, out_f32: bool = False):
