@@ -16,8 +16,8 @@
 // result does not depend on how its request's tokens were cut into steps or what shares the batch.
 #include "common.h"
 
-#define DR_LANES 8     // lanes that share a column of the state
-#define DR_TOKENS 16   // tokens staged in LDS at a time
+#define DR_LANES 16    // lanes that share a column of the state (a row of the wavefront's data paths)
+#define DR_TOKENS 16   // most tokens staged in LDS at a time
 #define DR_MAX_TAPS 16
 
 __device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + expf(-x)); }
@@ -104,21 +104,115 @@ __global__ void delta_tail_kernel(const T* __restrict__ proj, int ld, int taps, 
 }
 
 // --------------------------------------------------------------------------
-// The recurrence.  Workgroup (head, request, block of value columns); thread (column, lane):
-// the lane holds rows 4 * (lane + DR_LANES * n) + e of its column, n < NQ, e < 4.
+// The recurrence.  Workgroup (head, request, block of value columns); a column of the state is
+// owned by DR_LANES neighbouring lanes: lane holds rows 4 * (lane + DR_LANES * n) + e, n < NQ,
+// e < 4.  Per token, with the decayed column sd = g * s:
+//     dot = k . sd,  qs = q . sd   (one round of sums through the lanes for both)
+//     u = beta * (v - dot);  s = sd + k * u;  o = qs + u * (q . k)
+// (o = q . s written out: the read-out sees the token's own write).  q . k does not depend on
+// the column but costs little beside the other two sums.  The tokens' rows come through LDS
+// in chunks: DR_LOADERS threads of the workgroup do nothing but move the next chunk in while
+// the others compute this one, and meet them at a barrier a chunk.
+// The sums through the lanes use the lanes' own data paths (no LDS): partners exchange and
+// add, so every lane ends with the same bits, in an order that depends on nothing.
 // --------------------------------------------------------------------------
-template <int NQ>
-__global__ __launch_bounds__(NQ > 4 ? 256 : 1024) void delta_rule_kernel(
+__device__ __forceinline__ float dpp_quad_xor1(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float dpp_quad_xor2(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float dpp_half_mirror(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float dpp_row_mirror(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, true));
+}
+// the sum over the 16 lanes of a row, in every lane
+__device__ __forceinline__ float row_sum16(float v) {
+  v += dpp_quad_xor1(v);
+  v += dpp_quad_xor2(v);
+  v += dpp_half_mirror(v);
+  v += dpp_row_mirror(v);
+  return v;
+}
+
+// Rows of tokens t0 .. t0 + nt - 1 into a buffer [nt][q | k | decay (dkp each) | v (cols) | beta | padding], by
+// `nmove` threads of which this is `me`.  Several loads are in flight a thread before the first is stored.
+// VEC: the three long pieces move 16 bytes at a time (the caller found sizes and offsets to be multiples of 4).
+template <bool VEC>
+__device__ __forceinline__ void delta_move_rows(float* buf, const float* __restrict__ rec, int ld_rec, int t0, int nt,
+                                                int me, int nmove, int row_floats, int dkp, int dk, int dv, int cols,
+                                                int col0, int q_off, int k_off, int g_off, int v_off, int b_off) {
+  constexpr int B = 8;
+  if constexpr (VEC) {
+    const int per_row = 3 * dkp / 4;
+    for (int x0 = me; x0 < nt * per_row; x0 += B * nmove) {
+      float4 v[B];
+#pragma unroll
+      for (int j = 0; j < B; ++j) {
+        const int x = x0 + j * nmove;
+        v[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (x < nt * per_row) {
+          const int tt = x / per_row, rem = x % per_row, which = rem / (dkp / 4), i = 4 * (rem % (dkp / 4));
+          if (i < dk)
+            v[j] = *(const float4*)(rec + (size_t)(t0 + tt) * ld_rec + (which == 0 ? q_off : (which == 1 ? k_off : g_off)) + i);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < B; ++j) {
+        const int x = x0 + j * nmove;
+        if (x < nt * per_row) *(float4*)(buf + (x / per_row) * row_floats + 4 * (x % per_row)) = v[j];
+      }
+    }
+  }
+  const int first = VEC ? 3 * dkp : 0;  // what is left to move one by one
+  const int per_row = row_floats - first;
+  for (int x0 = me; x0 < nt * per_row; x0 += B * nmove) {
+    float v[B];
+#pragma unroll
+    for (int j = 0; j < B; ++j) {
+      const int x = x0 + j * nmove;
+      v[j] = 0.f;
+      if (x < nt * per_row) {
+        const int tt = x / per_row, rem = first + x % per_row;
+        const float* row = rec + (size_t)(t0 + tt) * ld_rec;
+        if (rem < 3 * dkp) {
+          const int which = rem / dkp, i = rem % dkp;
+          if (i < dk) v[j] = row[(which == 0 ? q_off : (which == 1 ? k_off : g_off)) + i];
+        } else if (rem < 3 * dkp + cols) {
+          const int c = rem - 3 * dkp;
+          if (col0 + c < dv) v[j] = row[v_off + col0 + c];
+        } else if (rem == 3 * dkp + cols) {
+          v[j] = row[b_off];
+        }
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < B; ++j) {
+      const int x = x0 + j * nmove;
+      if (x < nt * per_row) buf[(x / per_row) * row_floats + first + x % per_row] = v[j];
+    }
+  }
+}
+
+#define DR_LOADERS 128  // threads of a workgroup that only move the next chunk's rows into LDS
+
+template <int NQ, bool VEC>
+__global__ __launch_bounds__(NQ > 2 ? 384 : 1024) void delta_rule_kernel(
     const float* __restrict__ rec, int ld_rec, float* __restrict__ state, size_t state_stride,
     const int* __restrict__ q_start, const int* __restrict__ slots, float* __restrict__ o, int H, int G,
-    int dk, int dv, int cols) {
-  extern __shared__ __align__(16) float stage[];  // [DR_TOKENS][3][dkp] q, k, decay; [DR_TOKENS][cols] v; [DR_TOKENS] beta
+    int dk, int dv, int cols, int tok) {
+  // two buffers of [tok][3][dkp] q, k, decay; [tok][cols] v; [tok] beta
+  extern __shared__ __align__(16) float stage[];
   const int h = blockIdx.x, r = blockIdx.y;
   const int col0 = blockIdx.z * cols;
-  const int lane = threadIdx.x % DR_LANES;
-  const int col = col0 + threadIdx.x / DR_LANES;
-  const bool live = col < dv;
-  const int dkp = NQ * DR_LANES * 4;  // dk rounded up to what the lanes of a column hold
+  const int ncompute = cols * DR_LANES;
+  const bool loader = (int)threadIdx.x >= ncompute;
+  const int lane = threadIdx.x % DR_LANES, grp = threadIdx.x / DR_LANES;
+  const int col = col0 + grp;
+  const bool live = !loader && col < dv;
+  constexpr int dkp = NQ * DR_LANES * 4;  // dk rounded up to what the lanes of a column hold
   const int gk = h / (H / G);
   const int first = q_start[r], last = q_start[r + 1];
   float* s_col = state + (size_t)slots[r] * state_stride + ((size_t)h * dv + (live ? col : 0)) * dk;
@@ -132,62 +226,58 @@ __global__ __launch_bounds__(NQ > 4 ? 256 : 1024) void delta_rule_kernel(
       s[n][e] = (live && i < dk) ? s_col[i] : 0.f;
     }
 
-  float* sq = stage;
-  float* sv = stage + DR_TOKENS * 3 * dkp;
-  float* sb = sv + DR_TOKENS * cols;
+  const int row_floats = 3 * dkp + (cols + 1 + 3) / 4 * 4;
+  const int buf_floats = tok * row_floats;
   const int q_off = gk * dk, k_off = G * dk + gk * dk, v_off = 2 * G * dk + h * dv;
   const int g_off = 2 * G * dk + H * dv + h * dk, b_off = 2 * G * dk + H * dv + H * dk + h;
 
-  for (int t0 = first; t0 < last; t0 += DR_TOKENS) {
-    const int nt = min(DR_TOKENS, last - t0);
-    __syncthreads();  // the chunk before is consumed
-    for (int x = threadIdx.x; x < nt * dkp; x += blockDim.x) {
-      const int tt = x / dkp, i = x % dkp;
-      const float* row = rec + (size_t)(t0 + tt) * ld_rec;
-      const bool in = i < dk;
-      sq[(tt * 3 + 0) * dkp + i] = in ? row[q_off + i] : 0.f;
-      sq[(tt * 3 + 1) * dkp + i] = in ? row[k_off + i] : 0.f;
-      sq[(tt * 3 + 2) * dkp + i] = in ? row[g_off + i] : 0.f;
-    }
-    for (int x = threadIdx.x; x < nt * cols; x += blockDim.x) {
-      const int tt = x / cols, c = x % cols;
-      sv[x] = (col0 + c < dv) ? rec[(size_t)(t0 + tt) * ld_rec + v_off + col0 + c] : 0.f;
-    }
-    for (int x = threadIdx.x; x < nt; x += blockDim.x) sb[x] = rec[(size_t)(t0 + x) * ld_rec + b_off];
-    __syncthreads();
-    for (int tt = 0; tt < nt; ++tt) {
-      const float4* q4 = (const float4*)(sq + (tt * 3 + 0) * dkp);
-      const float4* k4 = (const float4*)(sq + (tt * 3 + 1) * dkp);
-      const float4* g4 = (const float4*)(sq + (tt * 3 + 2) * dkp);
-      float kk[NQ][4];
-      float dot = 0.f;
+#define move(BUF, T0, NT, ME, NMOVE) \
+  delta_move_rows<VEC>(BUF, rec, ld_rec, T0, NT, ME, NMOVE, row_floats, dkp, dk, dv, cols, col0, q_off, k_off, g_off, v_off, b_off)
+  if (first < last) move(stage, first, min(tok, last - first), threadIdx.x, blockDim.x);
+  __syncthreads();
+  int chunk = 0;
+#pragma unroll 1
+  for (int t0 = first; t0 < last; t0 += tok, ++chunk) {
+    const int nt = min(tok, last - t0);
+    const float* buf = stage + (chunk & 1) * buf_floats;
+    if (loader) {
+      const int next = t0 + tok;
+      if (next < last) move(stage + ((chunk + 1) & 1) * buf_floats, next, min(tok, last - next), threadIdx.x - ncompute, DR_LOADERS);
+    } else {
+#pragma unroll 1
+      for (int tt = 0; tt < nt; ++tt) {
+        const float* row = buf + tt * row_floats;
+        const float4* q4 = (const float4*)row;
+        const float4* k4 = (const float4*)(row + dkp);
+        const float4* g4 = (const float4*)(row + 2 * dkp);
+        float kk[NQ][4];
+        float dot[2] = {0.f, 0.f}, qs[2] = {0.f, 0.f}, kq[2] = {0.f, 0.f};
 #pragma unroll
-      for (int n = 0; n < NQ; ++n) {
-        const float4 g = g4[lane + DR_LANES * n], k = k4[lane + DR_LANES * n];
-        kk[n][0] = k.x; kk[n][1] = k.y; kk[n][2] = k.z; kk[n][3] = k.w;
-        s[n][0] *= g.x; s[n][1] *= g.y; s[n][2] *= g.z; s[n][3] *= g.w;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) dot = fmaf(kk[n][e], s[n][e], dot);
-      }
-#pragma unroll
-      for (int m = 1; m < DR_LANES; m <<= 1) dot += __shfl_xor(dot, m, TK_WAVE);
-      const float u = sb[tt] * (sv[tt * cols + threadIdx.x / DR_LANES] - dot);
-      float od = 0.f;
-#pragma unroll
-      for (int n = 0; n < NQ; ++n) {
-        const float4 q = q4[lane + DR_LANES * n];
-        const float qq[4] = {q.x, q.y, q.z, q.w};
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          s[n][e] = fmaf(kk[n][e], u, s[n][e]);
-          od = fmaf(qq[e], s[n][e], od);
+        for (int n = 0; n < NQ; ++n) {
+          const float4 g = g4[lane + DR_LANES * n], k = k4[lane + DR_LANES * n], q = q4[lane + DR_LANES * n];
+          kk[n][0] = k.x; kk[n][1] = k.y; kk[n][2] = k.z; kk[n][3] = k.w;
+          s[n][0] *= g.x; s[n][1] *= g.y; s[n][2] *= g.z; s[n][3] *= g.w;
+          dot[0] = fmaf(k.x, s[n][0], dot[0]); dot[1] = fmaf(k.y, s[n][1], dot[1]);
+          dot[0] = fmaf(k.z, s[n][2], dot[0]); dot[1] = fmaf(k.w, s[n][3], dot[1]);
+          qs[0] = fmaf(q.x, s[n][0], qs[0]); qs[1] = fmaf(q.y, s[n][1], qs[1]);
+          qs[0] = fmaf(q.z, s[n][2], qs[0]); qs[1] = fmaf(q.w, s[n][3], qs[1]);
+          kq[0] = fmaf(q.x, k.x, kq[0]); kq[1] = fmaf(q.y, k.y, kq[1]);
+          kq[0] = fmaf(q.z, k.z, kq[0]); kq[1] = fmaf(q.w, k.w, kq[1]);
         }
-      }
+        const float d = row_sum16(dot[0] + dot[1]);
+        const float qsum = row_sum16(qs[0] + qs[1]);
+        const float kqsum = row_sum16(kq[0] + kq[1]);
+        const float u = row[3 * dkp + cols] * (row[3 * dkp + grp] - d);
 #pragma unroll
-      for (int m = 1; m < DR_LANES; m <<= 1) od += __shfl_xor(od, m, TK_WAVE);
-      if (live && lane == 0) o[(size_t)(t0 + tt) * H * dv + (size_t)h * dv + col] = od;
+        for (int n = 0; n < NQ; ++n)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) s[n][e] = fmaf(kk[n][e], u, s[n][e]);
+        if (live && lane == 0) o[(size_t)(t0 + tt) * H * dv + (size_t)h * dv + col] = fmaf(u, kqsum, qsum);
+      }
     }
+    __syncthreads();
   }
+#undef move
   if (live) {
 #pragma unroll
     for (int n = 0; n < NQ; ++n)
@@ -273,20 +363,30 @@ TK_API int tk_delta_rule(const float* rec, int ld_rec, float* state, size_t stat
   TK_REQUIRE(n_requests < 65536, "delta_rule: too many requests");
   if (n_requests == 0) return 0;
   int nq = (dk + DR_LANES * 4 - 1) / (DR_LANES * 4);
-  nq = nq <= 2 ? nq : (nq <= 4 ? 4 : (nq <= 8 ? 8 : 16));  // the kernel's instances
-  TK_REQUIRE(nq <= 4 || cols * DR_LANES <= 256, "delta_rule: key size %d takes at most %d columns a workgroup", dk,
-             256 / DR_LANES);
+  nq = nq <= 2 ? nq : (nq <= 4 ? 4 : 8);  // the kernel's instances
   const int dkp = nq * DR_LANES * 4;
-  const size_t smem = sizeof(float) * ((size_t)DR_TOKENS * 3 * dkp + (size_t)DR_TOKENS * cols + DR_TOKENS);
-  const dim3 grid(H, n_requests, (dv + cols - 1) / cols), block(cols * DR_LANES);
-#define DR_CASE(NQ)                                                                                       \
-  hipLaunchKernelGGL(delta_rule_kernel<NQ>, grid, block, smem, stream, rec, ld_rec, state, state_stride, \
-                     q_start, slots, o, H, G, dk, dv, cols)
+  const int threads = cols * DR_LANES + DR_LOADERS;
+  TK_REQUIRE(threads <= (nq > 2 ? 384 : 1024), "delta_rule: %d columns a workgroup are too many for key size %d", cols, dk);
+  const int row_floats = 3 * dkp + (cols + 1 + 3) / 4 * 4;
+  int tok = 8192 / row_floats;  // two buffers of 32 KB at most
+  tok = tok > DR_TOKENS ? DR_TOKENS : tok;
+  TK_REQUIRE(tok >= 1, "delta_rule: key size %d with %d columns a workgroup", dk, cols);
+  const size_t smem = sizeof(float) * 2 * (size_t)tok * row_floats;
+  const dim3 grid(H, n_requests, (dv + cols - 1) / cols), block(threads);
+  const bool vec = dk % 4 == 0 && (H * dv) % 4 == 0 && ld_rec % 4 == 0 && ((uintptr_t)rec & 15) == 0;
+#define DR_CASE(NQ)                                                                                              \
+  do {                                                                                                           \
+    if (vec)                                                                                                     \
+      hipLaunchKernelGGL((delta_rule_kernel<NQ, true>), grid, block, smem, stream, rec, ld_rec, state,           \
+                         state_stride, q_start, slots, o, H, G, dk, dv, cols, tok);                              \
+    else                                                                                                         \
+      hipLaunchKernelGGL((delta_rule_kernel<NQ, false>), grid, block, smem, stream, rec, ld_rec, state,          \
+                         state_stride, q_start, slots, o, H, G, dk, dv, cols, tok);                              \
+  } while (0)
   if (nq == 1) DR_CASE(1);
   else if (nq == 2) DR_CASE(2);
   else if (nq == 4) DR_CASE(4);
-  else if (nq == 8) DR_CASE(8);
-  else DR_CASE(16);
+  else DR_CASE(8);
 #undef DR_CASE
   TK_CHECK_LAUNCH("delta_rule");
   return 0;

@@ -1258,7 +1258,8 @@ def delta_state_size(heads: int, kv_heads: int, key_dim: int, value_dim: int, ta
 
 
 def delta_rec_width(heads: int, kv_heads: int, key_dim: int, value_dim: int) -> int:
-    return 2 * kv_heads * key_dim + heads * value_dim + heads * key_dim + heads
+    """Numbers a token's row of the recurrence's input holds (q | k | v | decay | beta), filled up to a multiple of 4."""
+    return -(-(2 * kv_heads * key_dim + heads * value_dim + heads * key_dim + heads) // 4) * 4
 
 
 def delta_prepare(
@@ -1309,11 +1310,13 @@ def delta_prepare(
 
 
 def delta_rule_columns(requests: int, heads: int, key_dim: int, value_dim: int) -> int:
-    """Value columns a workgroup of the recurrence owns: as many as still leave the chip a few
-    workgroups a compute unit (a column's arithmetic does not depend on the choice)."""
-    most = 128 if key_dim <= 128 else 32
-    cols = 8
-    while cols * 2 <= most and cols < value_dim and requests * heads * -(-value_dim // (cols * 2)) >= 1024:
+    """Value columns a workgroup of the recurrence owns (16 lanes a column): few, so that the
+    chip gets many small workgroups whose wavefronts each have a vector unit to themselves (a
+    token's chain of operations is what takes the time); more only when there are so many
+    workgroups that they queue up anyway.  A column's arithmetic does not depend on the choice."""
+    most = 32 if key_dim <= 128 else 16
+    cols = 8 if value_dim > 4 else 4
+    while cols * 2 <= most and cols < value_dim and requests * heads * -(-value_dim // cols) > 4096:
         cols *= 2
     return cols
 
