@@ -25,17 +25,27 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 #define AT_MAX_KM 8   // dk <= 256
 #define AT_MAX_VT 16  // dv <= 256
 
-template <typename T, int KM, int VT>
+// 8 (4) neighbouring elements of the storage type, moved as one: what a lane loads of a key (of the values)
+template <typename T>
+struct __align__(16) Raw8 { T v[8]; };
+template <typename T>
+struct __align__(sizeof(T) * 4) Raw4 { T v[4]; };
+
+// SPLIT: the four wavefronts of a workgroup share one tile and take its key steps in turn
+// (wavefront w the steps w, w + 4, ..); they add up through LDS, always in wavefront order.
+// For steps of few tiles (single decoded tokens), whose walks would else be one long chain each.
+template <typename T, int KM, int VT, bool SPLIT>
 __global__ __launch_bounds__(AT_WAVES * TK_WAVE) void attention_tile_f32_kernel(
     const T* __restrict__ q, int q_stride, T* __restrict__ out, int out_stride, const T* __restrict__ kcache,
     const T* __restrict__ vcache, const int* __restrict__ block_table, int table_stride,
     const int* __restrict__ q_start, const int* __restrict__ kv_len, const int* __restrict__ tile_req,
     const int* __restrict__ tile_row0, int nq, int nkv, int dk, int dv, int P, int window, float scale,
     const float* __restrict__ sink, int gg) {
+  extern __shared__ float merge[];  // SPLIT: [waves][16] maxima, [waves][16] sums, [waves][VT][4][64] weighted values
   const int lane = threadIdx.x & (TK_WAVE - 1), wave = threadIdx.x / TK_WAVE;
   const int group = nq / nkv;
   const int blocks_per_kv = group / gg;  // head blocks of gg heads
-  const int hb = blockIdx.y * AT_WAVES + wave;
+  const int hb = SPLIT ? blockIdx.y : blockIdx.y * AT_WAVES + wave;
   if (hb >= nkv * blocks_per_kv) return;
   const int kvh = hb / blocks_per_kv;
   const int head0 = kvh * group + (hb % blocks_per_kv) * gg;
@@ -57,6 +67,7 @@ __global__ __launch_bounds__(AT_WAVES * TK_WAVE) void attention_tile_f32_kernel(
   const int lo_tile = window > 0 ? max(0, pos0 - window + 1) : 0;
   const int* table = block_table + (size_t)r * table_stride;
   const int pieces = dk / 8;
+  const size_t key_page = key_page_elems(P, dk);
 
   // the column's query, piece c + 4 m
   float qv[KM][8];
@@ -74,21 +85,46 @@ __global__ __launch_bounds__(AT_WAVES * TK_WAVE) void attention_tile_f32_kernel(
   for (int t = 0; t < VT; ++t) o[t] = (v4f){0.f, 0.f, 0.f, 0.f};
   float m_run = -INFINITY, l_run = 0.f;  // l_run: this lane's share of the column's sum
 
-  for (int k0 = (lo_tile / 16) * 16; k0 <= last; k0 += 16) {
-    const int page = max(table[k0 / P], 0);
-    const int in_page = k0 % P;
-    // S^T = K Q^T: this lane feeds key k0 + col, pieces c + 4 m
-    const T* kbase = kcache + ((size_t)page * nkv + kvh) * key_page_elems(P, dk);
-    v4f s = (v4f){0.f, 0.f, 0.f, 0.f};
+  const int step = SPLIT ? 16 * AT_WAVES : 16;
+  int k0 = (lo_tile / 16) * 16 + (SPLIT ? 16 * wave : 0);
+  // this lane's pieces of key k0 + col: the step's keys are asked for a step ahead
+  Raw8<T> kr[KM];
+  if (k0 <= last) {
+    const T* kbase = kcache + ((size_t)max(table[k0 / P], 0) * nkv + kvh) * key_page;
 #pragma unroll
     for (int m = 0; m < KM; ++m) {
       const int piece = c + 4 * m;
-      float kk[8];
-      const T* src = kbase + key_offset(P, in_page + col, (piece < pieces ? piece : 0) * 8);
+      kr[m] = *(const Raw8<T>*)(kbase + key_offset(P, k0 % P + col, (piece < pieces ? piece : 0) * 8));
+    }
+  }
+#pragma unroll 1
+  for (; k0 <= last; k0 += step) {
+    const int page = max(table[k0 / P], 0);
+    const int in_page = k0 % P;
+    // the step's values (element 16 t + col of keys k0 + 4 c + i) and the next step's keys: asked for now
+    const T* vbase = vcache + ((size_t)page * nkv + kvh) * P * dv;
+    Raw4<T> vr[VT];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) kk[e] = piece < pieces ? to_f32<T>(src[e]) : 0.f;
+    for (int t = 0; t < VT; ++t)
+      if (16 * t < dv) vr[t] = *(const Raw4<T>*)(vbase + value_offset(dv, in_page + 4 * c, 16 * t + col));
+    Raw8<T> kn[KM];
+    const int k1 = k0 + step;
+    if (k1 <= last) {
+      const T* kbase = kcache + ((size_t)max(table[k1 / P], 0) * nkv + kvh) * key_page;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) s = __builtin_amdgcn_mfma_f32_16x16x4f32(kk[e], qv[m][e], s, 0, 0, 0);
+      for (int m = 0; m < KM; ++m) {
+        const int piece = c + 4 * m;
+        kn[m] = *(const Raw8<T>*)(kbase + key_offset(P, k1 % P + col, (piece < pieces ? piece : 0) * 8));
+      }
+    }
+    // S^T = K Q^T
+    v4f s = (v4f){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int m = 0; m < KM; ++m) {
+      const bool in = c + 4 * m < pieces;
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        s = __builtin_amdgcn_mfma_f32_16x16x4f32(in ? to_f32<T>(kr[m].v[e]) : 0.f, qv[m][e], s, 0, 0, 0);
     }
     // this lane now holds, for its column, keys k0 + 4 c + i
     float sc[4];
@@ -115,26 +151,55 @@ __global__ __launch_bounds__(AT_WAVES * TK_WAVE) void attention_tile_f32_kernel(
     }
     m_run = m_new;
     l_run = l_run * alpha + ((p[0] + p[1]) + (p[2] + p[3]));
-    // O^T += V^T P^T: this lane feeds value element 16 t + col of keys k0 + 4 c + i
-    const T* vbase = vcache + ((size_t)page * nkv + kvh) * P * dv;
+    // O^T += V^T P^T
 #pragma unroll
     for (int t = 0; t < VT; ++t) {
       if (16 * t < dv) {
-        const T* src = vbase + value_offset(dv, in_page + 4 * c, 16 * t + col);
-        float vv[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) vv[i] = to_f32<T>(src[i]);
         v4f acc = o[t] * alpha;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(vv[i], p[i], acc, 0, 0, 0);
+        for (int i = 0; i < 4; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(to_f32<T>(vr[t].v[i]), p[i], acc, 0, 0, 0);
         o[t] = acc;
       }
     }
+#pragma unroll
+    for (int m = 0; m < KM; ++m) kr[m] = kn[m];
   }
   // the column's sum, from the four lanes that share it (always in this order)
   float l = l_run;
   l += __shfl_xor(l, 16, TK_WAVE);
   l += __shfl_xor(l, 32, TK_WAVE);
+  if constexpr (SPLIT) {
+    float* sm = merge;
+    float* sl = merge + AT_WAVES * 16;
+    float* so = merge + 2 * AT_WAVES * 16;
+    if (c == 0) {
+      sm[wave * 16 + col] = m_run;
+      sl[wave * 16 + col] = l;
+    }
+#pragma unroll
+    for (int t = 0; t < VT; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) so[((wave * VT + t) * 4 + i) * TK_WAVE + lane] = o[t][i];
+    __syncthreads();
+    if (wave != 0) return;
+    float m_all = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < AT_WAVES; ++w) m_all = fmaxf(m_all, sm[w * 16 + col]);
+    l = 0.f;
+#pragma unroll
+    for (int t = 0; t < VT; ++t) o[t] = (v4f){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int w = 0; w < AT_WAVES; ++w) {
+      const float mw = sm[w * 16 + col];
+      const float f = (mw == -INFINITY) ? 0.f : expf(mw - m_all);
+      l = fmaf(sl[w * 16 + col], f, l);
+#pragma unroll
+      for (int t = 0; t < VT; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[t][i] = fmaf(so[((w * VT + t) * 4 + i) * TK_WAVE + lane], f, o[t][i]);
+    }
+    m_run = m_all;
+  }
   float keep = 1.f;
   if (sink && live) {
     // the sink joins the softmax like one more score: the maximum may rise to it
@@ -161,20 +226,29 @@ TK_API int tk_attention_tile_f32_fits(int nq, int nkv, int dk, int dv, int P) {
 }
 
 template <typename T, int KM, int VT>
-static void at_launch(dim3 grid, hipStream_t stream, const void* q, int q_stride, void* out, int out_stride,
+static void at_launch(dim3 grid, bool split, hipStream_t stream, const void* q, int q_stride, void* out, int out_stride,
                       const void* kcache, const void* vcache, const int* block_table, int table_stride,
                       const int* q_start, const int* kv_len, const int* tile_req, const int* tile_row0, int nq,
                       int nkv, int dk, int dv, int P, int window, float scale, const float* sink, int gg) {
-  hipLaunchKernelGGL((attention_tile_f32_kernel<T, KM, VT>), grid, dim3(AT_WAVES * TK_WAVE), 0, stream, (const T*)q,
-                     q_stride, (T*)out, out_stride, (const T*)kcache, (const T*)vcache, block_table, table_stride,
-                     q_start, kv_len, tile_req, tile_row0, nq, nkv, dk, dv, P, window, scale, sink, gg);
+  if (split) {
+    const size_t smem = sizeof(float) * AT_WAVES * (32 + (size_t)VT * 4 * TK_WAVE);
+    hipLaunchKernelGGL((attention_tile_f32_kernel<T, KM, VT, true>), grid, dim3(AT_WAVES * TK_WAVE), smem, stream,
+                       (const T*)q, q_stride, (T*)out, out_stride, (const T*)kcache, (const T*)vcache, block_table,
+                       table_stride, q_start, kv_len, tile_req, tile_row0, nq, nkv, dk, dv, P, window, scale, sink, gg);
+  } else {
+    hipLaunchKernelGGL((attention_tile_f32_kernel<T, KM, VT, false>), grid, dim3(AT_WAVES * TK_WAVE), 0, stream,
+                       (const T*)q, q_stride, (T*)out, out_stride, (const T*)kcache, (const T*)vcache, block_table,
+                       table_stride, q_start, kv_len, tile_req, tile_row0, nq, nkv, dk, dv, P, window, scale, sink, gg);
+  }
 }
 
+// split: the wavefronts of a workgroup share a tile's keys (see the kernel); the caller chooses it for steps of few
+// tiles.  It changes the order in which a token's keys are added up, nothing else.
 TK_API int tk_attention_tile_f32(int dt, const void* q, int q_stride, void* out, int out_stride, const void* kcache,
                                  const void* vcache, const int* block_table, int table_stride, const int* q_start,
                                  const int* kv_len, const int* tile_req, const int* tile_row0, int n_tiles, int nq,
                                  int nkv, int dk, int dv, int P, int window, float scale, const float* sink, int gg,
-                                 hipStream_t stream) {
+                                 int split, hipStream_t stream) {
   TK_REQUIRE(tk_attention_tile_f32_fits(nq, nkv, dk, dv, P), "attention_tile_f32: shape nq=%d nkv=%d dk=%d dv=%d P=%d not taken",
              nq, nkv, dk, dv, P);
   const int group = nq / nkv;
@@ -182,10 +256,11 @@ TK_API int tk_attention_tile_f32(int dt, const void* q, int q_stride, void* out,
   TK_REQUIRE(q_stride >= nq * dk && out_stride >= nq * dv, "attention_tile_f32: row strides too short");
   if (n_tiles <= 0) return 0;
   const int head_blocks = nkv * (group / gg);
-  const dim3 grid(n_tiles, (head_blocks + AT_WAVES - 1) / AT_WAVES);
-  TK_REQUIRE(grid.y < 65536, "attention_tile_f32: too many heads");
   const int km = (dk + 31) / 32, vt = dv / 16;
-#define AT_ARGS grid, stream, q, q_stride, out, out_stride, kcache, vcache, block_table, table_stride, q_start, kv_len, \
+  const bool sp = split && vt <= 8;  // the sums of a wider value head do not fit the local memory
+  const dim3 grid(n_tiles, sp ? head_blocks : (head_blocks + AT_WAVES - 1) / AT_WAVES);
+  TK_REQUIRE(grid.y < 65536, "attention_tile_f32: too many heads");
+#define AT_ARGS grid, sp, stream, q, q_stride, out, out_stride, kcache, vcache, block_table, table_stride, q_start, kv_len, \
                 tile_req, tile_row0, nq, nkv, dk, dv, P, window, scale, sink, gg
 #define AT_VT(T, KMV)                                      \
   do {                                                     \

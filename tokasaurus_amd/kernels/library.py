@@ -43,7 +43,7 @@ _SIGNATURES: dict[str, dict[str, list]] = {
         "tk_softcap": [_P, c_size_t, c_float, _P],
         "tk_qk_prepare": [c_int, _P, c_int, _P, _P, _P, c_int, _P, _P, c_float, _P, _P, _P] + [c_int] * 8 + [_P],
         "tk_attention_tile_f32": [c_int, _P, c_int, _P, c_int, _P, _P, _P, c_int, _P, _P, _P, _P] + [c_int] * 7
-        + [c_float, _P, c_int, _P],
+        + [c_float, _P, c_int, c_int, _P],
         "tk_attention_tile_f32_fits": [c_int] * 5,
         "tk_delta_prepare": [c_int, _P, c_int, c_int, _P, _P, c_int, _P, _P, _P, c_size_t, c_size_t, _P, _P, _P, _P]
         + [c_int] * 7 + [_P],

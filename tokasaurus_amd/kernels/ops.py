@@ -1208,6 +1208,9 @@ def attention_tile_f32_fits(nq: int, nkv: int, key_dim: int, value_dim: int, pag
     return bool(load("core").tk_attention_tile_f32_fits(nq, nkv, key_dim, value_dim, page_size))
 
 
+ATTENTION_TILE_SPLIT_BELOW = 2048  # (tile, head block) pairs of a step below which the wavefronts share tiles
+
+
 def attention_tile_heads(group: int, max_q_len: int) -> int:
     """Query heads of one kv head that share a tile of 16 columns: one for prompt portions (16
     tokens a tile), as many as the group has (the largest power of two that divides it, at most
@@ -1224,13 +1227,17 @@ def attention_tile_f32(
     q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, block_table: torch.Tensor, q_start: torch.Tensor,
     kv_len: torch.Tensor, tile_req: torch.Tensor, tile_row0: torch.Tensor, nq: int, nkv: int, key_dim: int,
     value_dim: int, page_size: int, heads_a_tile: int, window: int = 0, scale: float = 1.0,
-    sink: torch.Tensor | None = None,
+    sink: torch.Tensor | None = None, split: bool | None = None,
 ) -> torch.Tensor:
     """Attention in 32-bit arithmetic on the matrix cores: every token of the step over its
     request's pages; ``tile_req`` / ``tile_row0`` name each tile's request and its first token's
     row (a tile holds 16 / heads_a_tile neighbouring tokens of one request).  Window, scale,
-    value size and sinks as in ``paged_attention_generic``; returns [tokens, nq * value_dim]."""
+    value size and sinks as in ``paged_attention_generic``; returns [tokens, nq * value_dim].
+    ``split``: the four wavefronts of a workgroup share a tile and take its keys in turn (by
+    default when the step has so few tiles that their walks would leave the chip idle)."""
     _gpu(q, kcache, vcache, block_table, q_start, kv_len, tile_req, tile_row0, sink)
+    if split is None:
+        split = tile_req.numel() * nkv * ((nq // nkv) // int(heads_a_tile)) < ATTENTION_TILE_SPLIT_BELOW
     _need(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= nq * key_dim,
           "attention: q must be 2-d with unit inner stride and nq*d leading columns")
     for t, name in ((block_table, "block_table"), (q_start, "q_start"), (kv_len, "kv_len"), (tile_req, "tile_req"), (tile_row0, "tile_row0")):
@@ -1244,7 +1251,8 @@ def attention_tile_f32(
     call("tk_attention_tile_f32", dtype_code(q.dtype), q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0),
          kcache.data_ptr(), vcache.data_ptr(), block_table.data_ptr(), block_table.stride(0), q_start.data_ptr(),
          kv_len.data_ptr(), tile_req.data_ptr(), tile_row0.data_ptr(), tile_req.numel(), nq, nkv, key_dim, value_dim,
-         page_size, int(window), float(scale), sink.data_ptr() if sink is not None else None, int(heads_a_tile), _stream())
+         page_size, int(window), float(scale), sink.data_ptr() if sink is not None else None, int(heads_a_tile),
+         1 if split else 0, _stream())
     return out
 
 
