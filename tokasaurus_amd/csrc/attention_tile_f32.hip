@@ -85,37 +85,38 @@ __global__ __launch_bounds__(AT_WAVES * TK_WAVE) void attention_tile_f32_kernel(
   for (int t = 0; t < VT; ++t) o[t] = (v4f){0.f, 0.f, 0.f, 0.f};
   float m_run = -INFINITY, l_run = 0.f;  // l_run: this lane's share of the column's sum
 
+  // where this lane's pieces of a key and its values lie inside a page, for the page's first key: both offsets
+  // grow linearly with the key's place in the page (8 elements a key, dv a key)
+  int koff[KM], voff[VT];
+#pragma unroll
+  for (int m = 0; m < KM; ++m) koff[m] = (int)key_offset(P, col, (c + 4 * m < pieces ? c + 4 * m : 0) * 8);
+#pragma unroll
+  for (int t = 0; t < VT; ++t) voff[t] = (int)value_offset(dv, 4 * c, 16 * t < dv ? 16 * t + col : 0);
   const int step = SPLIT ? 16 * AT_WAVES : 16;
   int k0 = (lo_tile / 16) * 16 + (SPLIT ? 16 * wave : 0);
   // this lane's pieces of key k0 + col: the step's keys are asked for a step ahead
   Raw8<T> kr[KM];
   if (k0 <= last) {
-    const T* kbase = kcache + ((size_t)max(table[k0 / P], 0) * nkv + kvh) * key_page;
+    const T* kbase = kcache + ((size_t)max(table[k0 / P], 0) * nkv + kvh) * key_page + (k0 % P) * 8;
 #pragma unroll
-    for (int m = 0; m < KM; ++m) {
-      const int piece = c + 4 * m;
-      kr[m] = *(const Raw8<T>*)(kbase + key_offset(P, k0 % P + col, (piece < pieces ? piece : 0) * 8));
-    }
+    for (int m = 0; m < KM; ++m) kr[m] = *(const Raw8<T>*)(kbase + koff[m]);
   }
 #pragma unroll 1
   for (; k0 <= last; k0 += step) {
     const int page = max(table[k0 / P], 0);
     const int in_page = k0 % P;
     // the step's values (element 16 t + col of keys k0 + 4 c + i) and the next step's keys: asked for now
-    const T* vbase = vcache + ((size_t)page * nkv + kvh) * P * dv;
+    const T* vbase = vcache + ((size_t)page * nkv + kvh) * P * dv + in_page * dv;
     Raw4<T> vr[VT];
 #pragma unroll
     for (int t = 0; t < VT; ++t)
-      if (16 * t < dv) vr[t] = *(const Raw4<T>*)(vbase + value_offset(dv, in_page + 4 * c, 16 * t + col));
+      if (16 * t < dv) vr[t] = *(const Raw4<T>*)(vbase + voff[t]);
     Raw8<T> kn[KM];
     const int k1 = k0 + step;
     if (k1 <= last) {
-      const T* kbase = kcache + ((size_t)max(table[k1 / P], 0) * nkv + kvh) * key_page;
+      const T* kbase = kcache + ((size_t)max(table[k1 / P], 0) * nkv + kvh) * key_page + (k1 % P) * 8;
 #pragma unroll
-      for (int m = 0; m < KM; ++m) {
-        const int piece = c + 4 * m;
-        kn[m] = *(const Raw8<T>*)(kbase + key_offset(P, k1 % P + col, (piece < pieces ? piece : 0) * 8));
-      }
+      for (int m = 0; m < KM; ++m) kn[m] = *(const Raw8<T>*)(kbase + koff[m]);
     }
     // S^T = K Q^T
     v4f s = (v4f){0.f, 0.f, 0.f, 0.f};

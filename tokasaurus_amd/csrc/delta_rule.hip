@@ -25,57 +25,82 @@ __device__ __forceinline__ float sigmoid_f32(float x) { return 1.0f / (1.0f + ex
 __device__ __forceinline__ float softplus_f32(float x) { return x > 20.f ? x : log1pf(expf(x)); }
 
 // --------------------------------------------------------------------------
-// Before the recurrence: one workgroup a token.
+// Before the recurrence.  A token's work is cut into units, one a wavefront: a q head or a k head
+// (convolution, silu, unit norm), a v head (convolution, silu), a head's decays, and the write
+// strengths of all heads.
 //   proj row (T): [q | k | v] (channels) ... and the write strength's `heads` numbers at col_b
 //   a_pre (32-bit) [tokens, heads * dk]: the decay's projection before bias and softplus
 //   rec row (32-bit): [q: G*dk | k: G*dk | v: H*dv | decay: H*dk | beta: H]
+// FUSE_TAIL (every request of the step brings one token): the lane that convolves a channel also
+// moves the channel's tail on, which it alone reads; else the kernel below does it afterwards.
 // --------------------------------------------------------------------------
-template <typename T>
+#define DP_MAX_PER_LANE 8  // dk, dv <= 512
+
+template <typename T, bool FUSE_TAIL>
 __global__ __launch_bounds__(256) void delta_prepare_kernel(
     const T* __restrict__ proj, int ld, int col_b, const float* __restrict__ a_pre,
     const float* __restrict__ conv_w, int taps, const float* __restrict__ a_log,
-    const float* __restrict__ dt_bias, const float* __restrict__ state, size_t state_stride,
+    const float* __restrict__ dt_bias, float* __restrict__ state, size_t state_stride,
     size_t tail_off, const int* __restrict__ q_start, const int* __restrict__ token_req,
     const int* __restrict__ slots, float* __restrict__ rec, int ld_rec, int H, int G, int dk, int dv) {
-  extern __shared__ float act[];  // [channels] convolved and activated
   const int t = blockIdx.x;
-  const int r = token_req[t];
-  const int first = q_start[r];
-  const int local = t - first;
+  const int lane = threadIdx.x & (TK_WAVE - 1);
+  const int unit = blockIdx.y * (blockDim.x / TK_WAVE) + threadIdx.x / TK_WAVE;
+  const int n_units = 2 * G + 2 * H + 1;
+  if (unit >= n_units) return;
   const int C = 2 * G * dk + H * dv;
-  const float* tail = state + (size_t)slots[r] * state_stride + tail_off;
-  for (int c = threadIdx.x; c < C; c += blockDim.x) {
-    float acc = 0.f;
-    for (int j = 0; j < taps; ++j) {
-      const int src = local - (taps - 1) + j;
-      const float x = src >= 0 ? to_f32<T>(proj[(size_t)(first + src) * ld + c])
-                               : tail[(size_t)(src + taps - 1) * C + c];
-      acc = fmaf(conv_w[(size_t)c * taps + j], x, acc);
-    }
-    act[c] = silu_f32(acc);
-  }
-  __syncthreads();
   float* out = rec + (size_t)t * ld_rec;
-  const int lane = threadIdx.x & (TK_WAVE - 1), wave = threadIdx.x / TK_WAVE;
-  const int nwaves = blockDim.x / TK_WAVE;
-  const float q_scale = 1.0f / sqrtf((float)dk);
-  for (int head = wave; head < 2 * G; head += nwaves) {  // q heads, then k heads: unit vectors
-    const float* x = act + head * dk;
-    float ss = 0.f;
-    for (int i = lane; i < dk; i += TK_WAVE) ss = fmaf(x[i], x[i], ss);
-    ss = wave_sum(ss);
-    float inv = 1.0f / sqrtf(ss + 1e-6f);
-    if (head < G) inv *= q_scale;
-    for (int i = lane; i < dk; i += TK_WAVE) out[head * dk + i] = x[i] * inv;
-  }
   const int v_off = 2 * G * dk, decay_off = v_off + H * dv, beta_off = decay_off + H * dk;
-  for (int i = threadIdx.x; i < H * dv; i += blockDim.x) out[v_off + i] = act[v_off + i];
-  for (int i = threadIdx.x; i < H * dk; i += blockDim.x) {
-    const float rate = expf(a_log[i / dk]);
-    out[decay_off + i] = expf(-rate * softplus_f32(a_pre[(size_t)t * H * dk + i] + dt_bias[i]));
+  if (unit < 2 * G + H) {
+    // a head's channels through the convolution: q head, k head or v head
+    const bool is_v = unit >= 2 * G;
+    const int width = is_v ? dv : dk;
+    const int c0 = is_v ? v_off + (unit - 2 * G) * dv : unit * dk;
+    const int r = token_req[t];
+    const int first = q_start[r];
+    const int local = t - first;
+    float* tail = state + (size_t)slots[r] * state_stride + tail_off;
+    float y[DP_MAX_PER_LANE];
+    float ss = 0.f;
+#pragma unroll
+    for (int n = 0; n < DP_MAX_PER_LANE; ++n) {
+      const int i = lane + n * TK_WAVE;
+      y[n] = 0.f;
+      if (i < width) {
+        const int c = c0 + i;
+        float acc = 0.f;
+        for (int j = 0; j < taps; ++j) {
+          const int src = local - (taps - 1) + j;
+          const float x = src >= 0 ? to_f32<T>(proj[(size_t)(first + src) * ld + c])
+                                   : tail[(size_t)(src + taps - 1) * C + c];
+          acc = fmaf(conv_w[(size_t)c * taps + j], x, acc);
+          if (FUSE_TAIL && j >= 1) tail[(size_t)(j - 1) * C + c] = x;  // (local is 0: entry j - 1 was read a tap ago)
+        }
+        y[n] = silu_f32(acc);
+        ss = fmaf(y[n], y[n], ss);
+      }
+    }
+    float mul = 1.f;
+    if (!is_v) {  // unit vectors; the queries also times dk^-1/2
+      mul = 1.0f / sqrtf(wave_sum(ss) + 1e-6f);
+      if (unit < G) mul *= 1.0f / sqrtf((float)dk);
+    }
+#pragma unroll
+    for (int n = 0; n < DP_MAX_PER_LANE; ++n) {
+      const int i = lane + n * TK_WAVE;
+      if (i < width) out[c0 + i] = y[n] * mul;
+    }
+  } else if (unit < 2 * G + 2 * H) {
+    const int h = unit - 2 * G - H;
+    const float rate = expf(a_log[h]);
+    for (int i = lane; i < dk; i += TK_WAVE) {
+      const int x = h * dk + i;
+      out[decay_off + x] = expf(-rate * softplus_f32(a_pre[(size_t)t * H * dk + x] + dt_bias[x]));
+    }
+  } else {
+    for (int i = lane; i < H; i += TK_WAVE)
+      out[beta_off + i] = sigmoid_f32(to_f32<T>(proj[(size_t)t * ld + col_b + i]));
   }
-  for (int i = threadIdx.x; i < H; i += blockDim.x)
-    out[beta_off + i] = sigmoid_f32(to_f32<T>(proj[(size_t)t * ld + col_b + i]));
 }
 
 // The convolutions' tails after the step: the last taps - 1 inputs of every request, taken
@@ -323,27 +348,33 @@ TK_API int tk_delta_prepare(int dt, const void* proj, int ld, int col_b, const f
   TK_REQUIRE(ld >= C && col_b >= 0 && col_b + H <= ld, "delta_prepare: row stride %d too short", ld);
   TK_REQUIRE(ld_rec >= C + H * dk + H, "delta_prepare: output stride %d too short", ld_rec);
   TK_REQUIRE(tail_off + (size_t)(taps - 1) * C <= state_stride, "delta_prepare: the state row is too short");
-  TK_REQUIRE((size_t)C * 4 <= 64 * 1024, "delta_prepare: %d channels do not fit the local memory", C);
+  TK_REQUIRE(dk <= DP_MAX_PER_LANE * TK_WAVE && dv <= DP_MAX_PER_LANE * TK_WAVE, "delta_prepare: head sizes %d, %d (at most %d)",
+             dk, dv, DP_MAX_PER_LANE * TK_WAVE);
   if (n_tokens == 0) return 0;
-  const size_t smem = sizeof(float) * (size_t)C;
+  const int units = 2 * G + 2 * H + 1;
+  const dim3 grid(n_tokens, (units + 3) / 4);
+  TK_REQUIRE(grid.y < 65536, "delta_prepare: too many heads");
+  // every request brings one token: the convolving lane moves its channel's tail on itself
+  const bool fuse_tail = n_tokens == n_requests && taps > 1;
+#define DP_LAUNCH(T, FUSE)                                                                                         \
+  hipLaunchKernelGGL((delta_prepare_kernel<T, FUSE>), grid, dim3(256), 0, stream, (const T*)proj, ld, col_b, a_pre, \
+                     conv_w, taps, a_log, dt_bias, state, state_stride, tail_off, q_start, token_req, slots, rec,  \
+                     ld_rec, H, G, dk, dv)
   if (dt == TK_F32) {
-    hipLaunchKernelGGL(delta_prepare_kernel<float>, dim3(n_tokens), dim3(256), smem, stream, (const float*)proj, ld,
-                       col_b, a_pre, conv_w, taps, a_log, dt_bias, state, state_stride, tail_off, q_start,
-                       token_req, slots, rec, ld_rec, H, G, dk, dv);
+    if (fuse_tail) DP_LAUNCH(float, true); else DP_LAUNCH(float, false);
   } else {
-    hipLaunchKernelGGL(delta_prepare_kernel<bf16_t>, dim3(n_tokens), dim3(256), smem, stream, (const bf16_t*)proj, ld,
-                       col_b, a_pre, conv_w, taps, a_log, dt_bias, state, state_stride, tail_off, q_start,
-                       token_req, slots, rec, ld_rec, H, G, dk, dv);
+    if (fuse_tail) DP_LAUNCH(bf16_t, true); else DP_LAUNCH(bf16_t, false);
   }
+#undef DP_LAUNCH
   TK_CHECK_LAUNCH("delta_prepare");
-  if (taps > 1 && n_requests > 0) {
+  if (taps > 1 && n_requests > 0 && !fuse_tail) {
     TK_REQUIRE(n_requests < 65536, "delta_prepare: too many requests");
-    const dim3 grid((C + 255) / 256, n_requests);
+    const dim3 tgrid((C + 255) / 256, n_requests);
     if (dt == TK_F32)
-      hipLaunchKernelGGL(delta_tail_kernel<float>, grid, dim3(256), 0, stream, (const float*)proj, ld, taps, state,
+      hipLaunchKernelGGL(delta_tail_kernel<float>, tgrid, dim3(256), 0, stream, (const float*)proj, ld, taps, state,
                          state_stride, tail_off, q_start, slots, C);
     else
-      hipLaunchKernelGGL(delta_tail_kernel<bf16_t>, grid, dim3(256), 0, stream, (const bf16_t*)proj, ld, taps, state,
+      hipLaunchKernelGGL(delta_tail_kernel<bf16_t>, tgrid, dim3(256), 0, stream, (const bf16_t*)proj, ld, taps, state,
                          state_stride, tail_off, q_start, slots, C);
     TK_CHECK_LAUNCH("delta_tail");
   }
