@@ -31,11 +31,11 @@ struct __align__(16) Raw8 { T v[8]; };
 template <typename T>
 struct __align__(sizeof(T) * 4) Raw4 { T v[4]; };
 
-// SPLIT: the four wavefronts of a workgroup share one tile and take its key steps in turn
-// (wavefront w the steps w, w + 4, ..); they add up through LDS, always in wavefront order.
+// SPLIT: the NW wavefronts of a workgroup share one tile and take its key steps in turn
+// (wavefront w the steps w, w + NW, ..); they add up through LDS, always in wavefront order.
 // For steps of few tiles (single decoded tokens), whose walks would else be one long chain each.
-template <typename T, int KM, int VT, bool SPLIT>
-__global__ __launch_bounds__(AT_WAVES * TK_WAVE) void attention_tile_f32_kernel(
+template <typename T, int KM, int VT, bool SPLIT, int NW>
+__global__ __launch_bounds__(NW * TK_WAVE) void attention_tile_f32_kernel(
     const T* __restrict__ q, int q_stride, T* __restrict__ out, int out_stride, const T* __restrict__ kcache,
     const T* __restrict__ vcache, const int* __restrict__ block_table, int table_stride,
     const int* __restrict__ q_start, const int* __restrict__ kv_len, const int* __restrict__ tile_req,
@@ -45,7 +45,7 @@ __global__ __launch_bounds__(AT_WAVES * TK_WAVE) void attention_tile_f32_kernel(
   const int lane = threadIdx.x & (TK_WAVE - 1), wave = threadIdx.x / TK_WAVE;
   const int group = nq / nkv;
   const int blocks_per_kv = group / gg;  // head blocks of gg heads
-  const int hb = SPLIT ? blockIdx.y : blockIdx.y * AT_WAVES + wave;
+  const int hb = SPLIT ? blockIdx.y : blockIdx.y * NW + wave;
   if (hb >= nkv * blocks_per_kv) return;
   const int kvh = hb / blocks_per_kv;
   const int head0 = kvh * group + (hb % blocks_per_kv) * gg;
@@ -92,7 +92,7 @@ __global__ __launch_bounds__(AT_WAVES * TK_WAVE) void attention_tile_f32_kernel(
   for (int m = 0; m < KM; ++m) koff[m] = (int)key_offset(P, col, (c + 4 * m < pieces ? c + 4 * m : 0) * 8);
 #pragma unroll
   for (int t = 0; t < VT; ++t) voff[t] = (int)value_offset(dv, 4 * c, 16 * t < dv ? 16 * t + col : 0);
-  const int step = SPLIT ? 16 * AT_WAVES : 16;
+  const int step = SPLIT ? 16 * NW : 16;
   int k0 = (lo_tile / 16) * 16 + (SPLIT ? 16 * wave : 0);
   // this lane's pieces of key k0 + col: the step's keys are asked for a step ahead
   Raw8<T> kr[KM];
@@ -171,8 +171,8 @@ __global__ __launch_bounds__(AT_WAVES * TK_WAVE) void attention_tile_f32_kernel(
   l += __shfl_xor(l, 32, TK_WAVE);
   if constexpr (SPLIT) {
     float* sm = merge;
-    float* sl = merge + AT_WAVES * 16;
-    float* so = merge + 2 * AT_WAVES * 16;
+    float* sl = merge + NW * 16;
+    float* so = merge + 2 * NW * 16;
     if (c == 0) {
       sm[wave * 16 + col] = m_run;
       sl[wave * 16 + col] = l;
@@ -185,12 +185,12 @@ __global__ __launch_bounds__(AT_WAVES * TK_WAVE) void attention_tile_f32_kernel(
     if (wave != 0) return;
     float m_all = -INFINITY;
 #pragma unroll
-    for (int w = 0; w < AT_WAVES; ++w) m_all = fmaxf(m_all, sm[w * 16 + col]);
+    for (int w = 0; w < NW; ++w) m_all = fmaxf(m_all, sm[w * 16 + col]);
     l = 0.f;
 #pragma unroll
     for (int t = 0; t < VT; ++t) o[t] = (v4f){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int w = 0; w < AT_WAVES; ++w) {
+    for (int w = 0; w < NW; ++w) {
       const float mw = sm[w * 16 + col];
       const float f = (mw == -INFINITY) ? 0.f : expf(mw - m_all);
       l = fmaf(sl[w * 16 + col], f, l);
@@ -232,12 +232,14 @@ static void at_launch(dim3 grid, bool split, hipStream_t stream, const void* q, 
                       const int* q_start, const int* kv_len, const int* tile_req, const int* tile_row0, int nq,
                       int nkv, int dk, int dv, int P, int window, float scale, const float* sink, int gg) {
   if (split) {
-    const size_t smem = sizeof(float) * AT_WAVES * (32 + (size_t)VT * 4 * TK_WAVE);
-    hipLaunchKernelGGL((attention_tile_f32_kernel<T, KM, VT, true>), grid, dim3(AT_WAVES * TK_WAVE), smem, stream,
+    // eight wavefronts a tile where their sums fit the local memory, else four
+    constexpr int NW = VT <= 4 ? 8 : 4;
+    const size_t smem = sizeof(float) * NW * (32 + (size_t)VT * 4 * TK_WAVE);
+    hipLaunchKernelGGL((attention_tile_f32_kernel<T, KM, VT, true, NW>), grid, dim3(NW * TK_WAVE), smem, stream,
                        (const T*)q, q_stride, (T*)out, out_stride, (const T*)kcache, (const T*)vcache, block_table,
                        table_stride, q_start, kv_len, tile_req, tile_row0, nq, nkv, dk, dv, P, window, scale, sink, gg);
   } else {
-    hipLaunchKernelGGL((attention_tile_f32_kernel<T, KM, VT, false>), grid, dim3(AT_WAVES * TK_WAVE), 0, stream,
+    hipLaunchKernelGGL((attention_tile_f32_kernel<T, KM, VT, false, AT_WAVES>), grid, dim3(AT_WAVES * TK_WAVE), 0, stream,
                        (const T*)q, q_stride, (T*)out, out_stride, (const T*)kcache, (const T*)vcache, block_table,
                        table_stride, q_start, kv_len, tile_req, tile_row0, nq, nkv, dk, dv, P, window, scale, sink, gg);
   }
