@@ -58,14 +58,15 @@ RECURRENT = {
     "residual_mult": 1.0,
     "layers": [delta_layer(1, 1, 72, 24, 1, 8, 8, ff=96), delta_layer(6, 2, 16, 16, 2, 24, 16)],
 }
-# only attention: a key size that is no multiple of 8, a window of one key, no grouping, no rotation in one layer
+# only attention: key sizes that are no multiples of 8 (one of them odd), a window of one key, no grouping, no rotation in one layer
 WINDOWS = {
     "architecture": "Kupuzen", "vocab": 200, "width": 80, "embedding": {"scale": 0.7}, "norm": {"eps": 1e-4},
     "residual_mult": 0.8, "logit_softcap": 50.0,
     "layers": [
         attention_layer(4, 4, 20, 12, 0.4, window=1, rot={"base": 50.0, "dims": 20}, ff=48),
+        attention_layer(3, 1, 7, 5, 0.6, window=11, rot={"base": 30.0, "dims": 6}),
         attention_layer(8, 2, 16, 32, 0.5, window=16, rot={"base": 1000.0, "dims": 4}),
-        attention_layer(8, 2, 16, 32, 0.35, window=5, kv_from=1, ff=48),
+        attention_layer(8, 2, 16, 32, 0.35, window=5, kv_from=2, ff=48),
         attention_layer(2, 1, 32, 8, 0.2, window=64, ff=32),
     ],
 }

@@ -158,4 +158,4 @@ def test_a_cache_that_another_layer_reads_keeps_the_wider_window():
     assert [s is not None for s in model.state_needs()] == [False, True, False, True, False]
     arch = architecture_of(WINDOWS)
     needs = build_model(arch, arch.config_from_dict(WINDOWS)).cache_needs()
-    assert [n.window for n in needs] == [1, 16, 16, 64]
+    assert [n.window for n in needs] == [1, 11, 16, 16, 64]

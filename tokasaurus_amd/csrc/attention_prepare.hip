@@ -51,17 +51,19 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
   }
   __syncthreads();  // the table of this token's angles is written
 
-  // queries, in place, a pair a thread
-  for (int i = threadIdx.x; i < nqe / 2; i += blockDim.x) {
-    const int e = (2 * i) % dk;
-    float u = to_f32<T>(row[2 * i]) * rq, v = to_f32<T>(row[2 * i + 1]) * rq;
+  // queries, in place, a pair of neighbours a thread (a head of odd size ends in a single element)
+  const int hp = (dk + 1) / 2;
+  for (int i = threadIdx.x; i < nq * hp; i += blockDim.x) {
+    const int e = 2 * (i % hp), x = (i / hp) * dk + e;
+    const bool two = e + 1 < dk;
+    float u = to_f32<T>(row[x]) * rq, v = two ? to_f32<T>(row[x + 1]) * rq : 0.f;
     if (q_weight) {
-      u *= q_weight[2 * i];
-      v *= q_weight[2 * i + 1];
+      u *= q_weight[x];
+      if (two) v *= q_weight[x + 1];
     }
     if (e < rot) rotate_pair(u, v, cs[e / 2], cs[half + e / 2], u, v);
-    row[2 * i] = from_f32<T>(u);
-    row[2 * i + 1] = from_f32<T>(v);
+    row[x] = from_f32<T>(u);
+    if (two) row[x + 1] = from_f32<T>(v);
   }
   if (!write_cache) return;
 
@@ -69,17 +71,18 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
   const int p = pos % P;
   const T* krow = row + nqe;
   const T* vrow = krow + nke;
-  for (int i = threadIdx.x; i < nke / 2; i += blockDim.x) {
-    const int h = (2 * i) / dk, e = (2 * i) % dk;
-    float u = to_f32<T>(krow[2 * i]) * rk, v = to_f32<T>(krow[2 * i + 1]) * rk;
+  for (int i = threadIdx.x; i < nkv * hp; i += blockDim.x) {
+    const int h = i / hp, e = 2 * (i % hp), x = h * dk + e;
+    const bool two = e + 1 < dk;
+    float u = to_f32<T>(krow[x]) * rk, v = two ? to_f32<T>(krow[x + 1]) * rk : 0.f;
     if (k_weight) {
-      u *= k_weight[2 * i];
-      v *= k_weight[2 * i + 1];
+      u *= k_weight[x];
+      if (two) v *= k_weight[x + 1];
     }
     if (e < rot) rotate_pair(u, v, cs[e / 2], cs[half + e / 2], u, v);
     T* dst = kcache + ((size_t)page * nkv + h) * key_page_elems(P, dk);
     dst[key_offset(P, p, e)] = from_f32<T>(u);
-    dst[key_offset(P, p, e + 1)] = from_f32<T>(v);
+    if (two) dst[key_offset(P, p, e + 1)] = from_f32<T>(v);
   }
   for (int i = threadIdx.x; i < nkv * dv; i += blockDim.x) {
     const int h = i / dv, e = i % dv;
@@ -92,7 +95,7 @@ TK_API int tk_qk_prepare(int dt, void* qkv, int row_stride, const int* positions
                          const float* k_weight, float eps, const float* freq, void* kcache, void* vcache,
                          int n_tokens, int nq, int nkv, int dk, int dv, int rot, int P, int write_cache,
                          hipStream_t stream) {
-  TK_REQUIRE(n_tokens >= 0 && nq > 0 && nkv >= 0 && dk > 0 && dk % 2 == 0 && dv > 0 && P > 0,
+  TK_REQUIRE(n_tokens >= 0 && nq > 0 && nkv >= 0 && dk > 0 && dv > 0 && P > 0,
              "qk_prepare: bad sizes tokens=%d nq=%d nkv=%d dk=%d dv=%d P=%d", n_tokens, nq, nkv, dk, dv, P);
   TK_REQUIRE(rot >= 0 && rot <= dk && rot % 2 == 0, "qk_prepare: %d rotated elements of a head of %d", rot, dk);
   TK_REQUIRE(rot == 0 || freq, "qk_prepare: a rotation needs its frequencies");
