@@ -86,6 +86,7 @@ def parse() -> argparse.Namespace:
                    help="instead of the decode steps: prefill and decode of this design at layer sizes of --design-sizes "
                         "beside the Llama shape of equal width, heads, feed-forward and layers (prints its own line)")
     p.add_argument("--design-sizes", default="1b,3b", help="which sizes of DESIGN_SIZES, comma separated")
+    p.add_argument("--design-only", action="store_true", help="the --design comparison without its Llama half (for profiles)")
     p.add_argument("--design-layers", type=int, default=8, help="layers of both models in the --design comparison")
     p.add_argument("--design-context", type=int, default=4096, help="context at which the --design decode steps end")
     p.add_argument("--portion", type=int, default=128)
@@ -372,6 +373,8 @@ def run_design(args) -> int:
         size = DESIGN_SIZES[name]
         configs = {"llama": dict(size["llama"], num_hidden_layers=args.design_layers),
                    args.design: kupuzen_like(size, args.design_layers)}
+        if args.design_only:
+            del configs["llama"]
         rec = {}
         for model, cfgd in configs.items():
             runner = build_runner(cfgd, args.dtype, max(batches) * ctx, max(batches), ctx, use_graphs=not args.eager)
@@ -388,7 +391,8 @@ def run_design(args) -> int:
             say(f"{name} {model}: {one}")
             del runner
             torch.cuda.empty_cache()
-        rec["ratio"] = {k: round(rec[args.design][k] / rec["llama"][k], 3) for k in rec["llama"] if k.endswith("tok_per_s")}
+        if not args.design_only:
+            rec["ratio"] = {k: round(rec[args.design][k] / rec["llama"][k], 3) for k in rec["llama"] if k.endswith("tok_per_s")}
         out["sizes"][name] = rec
     print(json.dumps(out))
     return 0
