@@ -118,24 +118,32 @@ __global__ __launch_bounds__(NW * TK_WAVE) void attention_tile_f32_kernel(
 #pragma unroll
       for (int m = 0; m < KM; ++m) kn[m] = *(const Raw8<T>*)(kbase + koff[m]);
     }
-    // S^T = K Q^T
+    // S^T = K Q^T (a piece beyond the head's size meets zeros of the query)
     v4f s = (v4f){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int m = 0; m < KM; ++m) {
-      const bool in = c + 4 * m < pieces;
+    for (int m = 0; m < KM; ++m)
 #pragma unroll
       for (int e = 0; e < 8; ++e)
-        s = __builtin_amdgcn_mfma_f32_16x16x4f32(in ? to_f32<T>(kr[m].v[e]) : 0.f, qv[m][e], s, 0, 0, 0);
-    }
+        s = __builtin_amdgcn_mfma_f32_16x16x4f32(to_f32<T>(kr[m].v[e]), qv[m][e], s, 0, 0, 0);
     // this lane now holds, for its column, keys k0 + 4 c + i
     float sc[4];
     float tmax = -INFINITY;
+    // a step that every column of the tile sees whole needs no masks (the same for all lanes)
+    const bool whole = k0 + 15 <= pos0 && (window <= 0 || last - k0 < window) && n_tok * gg == 16;
+    if (whole) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int kp = k0 + 4 * c + i;
-      const bool seen = live && kp <= pos && (window <= 0 || pos - kp < window);
-      sc[i] = seen ? s[i] * scale : -INFINITY;
-      tmax = fmaxf(tmax, sc[i]);
+      for (int i = 0; i < 4; ++i) {
+        sc[i] = s[i] * scale;
+        tmax = fmaxf(tmax, sc[i]);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int kp = k0 + 4 * c + i;
+        const bool seen = live && kp <= pos && (window <= 0 || pos - kp < window);
+        sc[i] = seen ? s[i] * scale : -INFINITY;
+        tmax = fmaxf(tmax, sc[i]);
+      }
     }
     tmax = fmaxf(tmax, __shfl_xor(tmax, 16, TK_WAVE));
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, TK_WAVE));
@@ -146,9 +154,10 @@ __global__ __launch_bounds__(NW * TK_WAVE) void attention_tile_f32_kernel(
 #pragma unroll
       for (int i = 0; i < 4; ++i) p[i] = 0.f;
     } else {
-      alpha = (m_run == -INFINITY) ? 0.f : expf(m_run - m_new);
+      // exp2 of the difference times log2(e): the hardware's own exponential (a masked score gives exp2(-inf) = 0)
+      alpha = exp2f((m_run - m_new) * 1.44269504088896341f);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) p[i] = (sc[i] == -INFINITY) ? 0.f : expf(sc[i] - m_new);
+      for (int i = 0; i < 4; ++i) p[i] = exp2f((sc[i] - m_new) * 1.44269504088896341f);
     }
     m_run = m_new;
     l_run = l_run * alpha + ((p[0] + p[1]) + (p[2] + p[3]));
