@@ -70,7 +70,21 @@ WINDOWS = {
         attention_layer(2, 1, 32, 8, 0.2, window=64, ff=32),
     ],
 }
-CONFIGS = {"mixed": MIXED, "recurrent": RECURRENT, "windows": WINDOWS}
+# sizes that fit nothing: a width, feed-forward sizes, a vocabulary and low ranks that are no multiples of 8 (or of 2),
+# delta-rule heads of 48 x 20 and 136 x 12 with grouping, 6 taps, large attention heads without grouping, two
+# layers that read one owner's keys, a rotation of the whole head with scaling
+AWKWARD = {
+    "architecture": "Kupuzen", "vocab": 131, "width": 100, "embedding": {"scale": 1.5}, "norm": {"eps": 1e-6},
+    "residual_mult": 0.4, "logit_softcap": 12.0,
+    "layers": [
+        delta_layer(3, 1, 48, 20, 6, 10, 7, ff=75),
+        attention_layer(2, 2, 128, 128, 0.09, window=50, rot={"base": 5000.0, "dims": 128, "scaling": {"factor": 2.0, "low": 1.0, "high": 2.0, "original": 16}}, ff=52),
+        attention_layer(2, 2, 128, 128, 0.1, window=70, rot={"base": 5000.0, "dims": 128, "scaling": {"factor": 2.0, "low": 1.0, "high": 2.0, "original": 16}}, kv_from=1),
+        delta_layer(2, 1, 136, 12, 2, 5, 9),
+        attention_layer(2, 2, 128, 128, 0.08, window=3, rot={"base": 5000.0, "dims": 128, "scaling": {"factor": 2.0, "low": 1.0, "high": 2.0, "original": 16}}, kv_from=1, ff=33),
+    ],
+}
+CONFIGS = {"mixed": MIXED, "recurrent": RECURRENT, "windows": WINDOWS, "awkward": AWKWARD}
 
 
 def make_folder(folder: Path, config: dict, seed: int, edits: dict | None = None) -> Path:
