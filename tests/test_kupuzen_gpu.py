@@ -60,6 +60,9 @@ SINGLE_LAYERS = {
     "attention_matrix_core_sizes_odd_group": attention_layer(6, 2, 8, 16, 0.3, rot={"base": 100.0, "dims": 8}),
     "delta": delta_layer(4, 2, 16, 24, 4, 8, 16),
     "delta_wide_key": delta_layer(2, 1, 136, 8, 2, 8, 8, ff=32),
+    "delta_sizes_of_a_large_model": delta_layer(2, 1, 128, 128, 4, 16, 16),
+    "delta_key_of_96": delta_layer(4, 4, 96, 64, 3, 8, 8),
+    "attention_sizes_of_a_large_model": attention_layer(8, 2, 64, 64, 0.125, window=24, rot={"base": 500000.0, "dims": 64}),
     "feed_forward_beside_attention": attention_layer(1, 1, 8, 8, 1.0, window=2, ff=72),
 }
 
