@@ -94,29 +94,57 @@ __global__ __launch_bounds__(NW * TK_WAVE) void attention_tile_f32_kernel(
   for (int t = 0; t < VT; ++t) voff[t] = (int)value_offset(dv, 4 * c, 16 * t < dv ? 16 * t + col : 0);
   const int step = SPLIT ? 16 * NW : 16;
   int k0 = (lo_tile / 16) * 16 + (SPLIT ? 16 * wave : 0);
-  // this lane's pieces of key k0 + col: the step's keys are asked for a step ahead
+  // The pages of this wavefront's steps, 64 steps at a time: lane j asks for the page of step `base + j`, and a
+  // step reads its page's number from that lane.  So no load of keys or values waits for a load of a page number.
+  const int k_first = k0;
+  int pv = 0;
+#define AT_PAGES(BASE)                                                  \
+  do {                                                                  \
+    const int kj = k_first + ((BASE) + lane) * step;                    \
+    pv = kj <= last ? max(table[kj / P], 0) : 0;                        \
+  } while (0)
+  AT_PAGES(0);
+  // this lane's pieces of key k0 + col and its values (element 16 t + col of keys k0 + 4 c + i); the keys are
+  // asked for a step ahead, and (SPLIT, where nothing else hides the wait) the values too
   Raw8<T> kr[KM];
+  Raw4<T> vr[VT];
   if (k0 <= last) {
-    const T* kbase = kcache + ((size_t)max(table[k0 / P], 0) * nkv + kvh) * key_page + (k0 % P) * 8;
+    const int page = __builtin_amdgcn_readlane(pv, 0);
+    const T* kbase = kcache + ((size_t)page * nkv + kvh) * key_page + (k0 % P) * 8;
 #pragma unroll
     for (int m = 0; m < KM; ++m) kr[m] = *(const Raw8<T>*)(kbase + koff[m]);
-  }
-#pragma unroll 1
-  for (; k0 <= last; k0 += step) {
-    const int page = max(table[k0 / P], 0);
-    const int in_page = k0 % P;
-    // the step's values (element 16 t + col of keys k0 + 4 c + i) and the next step's keys: asked for now
-    const T* vbase = vcache + ((size_t)page * nkv + kvh) * P * dv + in_page * dv;
-    Raw4<T> vr[VT];
+    if constexpr (SPLIT) {
+      const T* vbase = vcache + ((size_t)page * nkv + kvh) * P * dv + (k0 % P) * dv;
 #pragma unroll
-    for (int t = 0; t < VT; ++t)
-      if (16 * t < dv) vr[t] = *(const Raw4<T>*)(vbase + voff[t]);
+      for (int t = 0; t < VT; ++t)
+        if (16 * t < dv) vr[t] = *(const Raw4<T>*)(vbase + voff[t]);
+    }
+  }
+  int j = 0;
+#pragma unroll 1
+  for (; k0 <= last; k0 += step, ++j) {
+    if constexpr (!SPLIT) {
+      const int page = __builtin_amdgcn_readlane(pv, j & 63);
+      const T* vbase = vcache + ((size_t)page * nkv + kvh) * P * dv + (k0 % P) * dv;
+#pragma unroll
+      for (int t = 0; t < VT; ++t)
+        if (16 * t < dv) vr[t] = *(const Raw4<T>*)(vbase + voff[t]);
+    }
     Raw8<T> kn[KM];
+    Raw4<T> vn[VT];
     const int k1 = k0 + step;
     if (k1 <= last) {
-      const T* kbase = kcache + ((size_t)max(table[k1 / P], 0) * nkv + kvh) * key_page + (k1 % P) * 8;
+      if (((j + 1) & 63) == 0) AT_PAGES(j + 1);
+      const int page1 = __builtin_amdgcn_readlane(pv, (j + 1) & 63);
+      const T* kbase = kcache + ((size_t)page1 * nkv + kvh) * key_page + (k1 % P) * 8;
 #pragma unroll
       for (int m = 0; m < KM; ++m) kn[m] = *(const Raw8<T>*)(kbase + koff[m]);
+      if constexpr (SPLIT) {
+        const T* vbase = vcache + ((size_t)page1 * nkv + kvh) * P * dv + (k1 % P) * dv;
+#pragma unroll
+        for (int t = 0; t < VT; ++t)
+          if (16 * t < dv) vn[t] = *(const Raw4<T>*)(vbase + voff[t]);
+      }
     }
     // S^T = K Q^T (a piece beyond the head's size meets zeros of the query)
     v4f s = (v4f){0.f, 0.f, 0.f, 0.f};
@@ -173,7 +201,12 @@ __global__ __launch_bounds__(NW * TK_WAVE) void attention_tile_f32_kernel(
     }
 #pragma unroll
     for (int m = 0; m < KM; ++m) kr[m] = kn[m];
+    if constexpr (SPLIT) {
+#pragma unroll
+      for (int t = 0; t < VT; ++t) vr[t] = vn[t];
+    }
   }
+#undef AT_PAGES
   // the column's sum, from the four lanes that share it (always in this order)
   float l = l_run;
   l += __shfl_xor(l, 16, TK_WAVE);
