@@ -214,8 +214,9 @@ def test_first_tokens_of_a_sequence(kupuzen_folders):
             compare_rows(run_steps(runner, portions(rid, toks, [1])), plain, TOL["float32"])
 
 
+@pytest.mark.parametrize("name", ["mixed", "recurrent"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_greedy_generation_through_the_engine(kupuzen_folders, dtype):
+def test_greedy_generation_through_the_engine(kupuzen_folders, dtype, name):
     """``Engine.generate``: the scheduler cuts prompts into portions beside decoding requests;
     the tokens are the plain model's greedy tokens (in bfloat16: each token is, for the plain
     logits of its own history, within rounding of the best)."""
@@ -223,7 +224,7 @@ def test_greedy_generation_through_the_engine(kupuzen_folders, dtype):
     from tokasaurus_amd.engine.engine import Engine
     from tokasaurus_amd.sampling import SamplingParams
 
-    folder, vocab = kupuzen_folders["mixed"], MIXED["vocab"]
+    folder, vocab = kupuzen_folders[name], CONFIGS[name]["vocab"]  # "recurrent" keeps no keys at all: no page is ever counted
     prompts = [random_tokens(n, vocab, 10 + n) for n in (5, 40, 23, 1, 64)]
     engine = Engine(EngineConfig(model=str(folder), dtype=dtype, page_size=PAGE, kv_cache_num_tokens=512, max_seqs_per_forward=3,
                                  max_tokens_per_forward=24, allocator_sanity_checks=True))
