@@ -241,3 +241,58 @@ def test_greedy_generation_through_the_engine(kupuzen_folders, dtype, name):
                 assert float(logits.max() - logits[tok]) < 0.05 * float(logits.std()) + 0.05
             ids.append(tok)
     assert engine.runner.manager.requests == {}
+
+
+def test_command_line_and_trace_replay(kupuzen_folders, tmp_path):
+    """``bin/toka`` generates from a Kupuzen folder (also from a config.json alone, with random weights, where the
+    low ranks that no checkpoint gives come from the file or a default), and ``bin/trace_run`` replays given tokens
+    step by step: its logits are the plain model's."""
+    import os
+    import subprocess
+    import sys
+
+    import numpy as np
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    folder, vocab = kupuzen_folders["mixed"], MIXED["vocab"]
+    prompts = [random_tokens(9, vocab, 1), random_tokens(20, vocab, 2)]
+    proc = subprocess.run([sys.executable, os.path.join(root, "bin", "toka"), f"model={folder}", "dtype=float32", f"page_size={PAGE}",
+                           "kv_cache_num_tokens=256", f"prompt_ids=({json.dumps(prompts)})", "max_tokens=5", "ignore_eos=T"],
+                          capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    lines = [json.loads(l) for l in proc.stdout.splitlines() if l.strip()]
+    cfg, w = load_plain(folder)
+    for prompt, line in zip(prompts, lines):
+        ids = list(prompt)
+        for tok in line["tokens"]:
+            assert tok == int(pk.forward(cfg, w, ids)[-1].argmax())
+            ids.append(tok)
+    bare = copy.deepcopy(RECURRENT)
+    for layer in bare["layers"]:
+        del layer["mixer"]["decay_rank"], layer["mixer"]["gate_rank"]
+    model = tmp_path / "fresh"
+    model.mkdir()
+    (model / "config.json").write_text(json.dumps(bare))
+    proc = subprocess.run([sys.executable, os.path.join(root, "bin", "toka"), f"model={model}", "random_weights=T", "seed=5",
+                           "dtype=bfloat16", "num_prompts=2", "prompt_len=7", "max_tokens=3"], capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert (model / "model.safetensors").is_file() and len(proc.stdout.splitlines()) == 2
+    # the replay tool: two requests, portions beside single tokens, the first ended before the second
+    a, b = random_tokens(21, vocab, 3), random_tokens(40, vocab, 4)
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": a[:17], "want": [0, 16]}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": a[17:18], "want": [0]}, {"id": "b", "tokens": b[:33], "want": [32]}], "end": []},
+        {"step": 2, "entries": [{"id": "b", "tokens": b[33:35], "want": []}, {"id": "a", "tokens": a[18:], "want": [2]}], "end": ["a"]},
+        {"step": 3, "entries": [{"id": "b", "tokens": b[35:], "want": [4]}], "end": ["b"]},
+    ]
+    out = tmp_path / "out"
+    proc = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", str(folder), "--dtype", "float32",
+                           "--out", str(out), "--max-tokens", "128"], input="\n".join(json.dumps(s) for s in steps) + "\n",
+                          capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == [f"done {i}" for i in range(4)]
+    plain = plain_rows(folder, {"a": a, "b": b})
+    want = {0: [("a", 0), ("a", 16)], 1: [("a", 17), ("b", 32)], 2: [("a", 20)], 3: [("b", 39)]}
+    for step, rows in want.items():
+        got = torch.from_numpy(np.fromfile(out / f"{step}.f32", dtype="<f4").reshape(len(rows), vocab).copy())
+        compare_rows({key: got[i] for i, key in enumerate(rows)}, plain, TOL["float32"])
