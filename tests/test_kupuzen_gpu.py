@@ -62,6 +62,9 @@ SINGLE_LAYERS = {
     "delta_wide_key": delta_layer(2, 1, 136, 8, 2, 8, 8, ff=32),
     "delta_sizes_of_a_large_model": delta_layer(2, 1, 128, 128, 4, 16, 16),
     "delta_key_of_96": delta_layer(4, 4, 96, 64, 3, 8, 8),
+    "attention_largest_heads_of_the_matrix_core_kernel": attention_layer(2, 1, 256, 256, 0.06, window=40, rot={"base": 1e4, "dims": 96}),
+    "attention_heads_beyond_it": attention_layer(2, 2, 264, 16, 0.06, window=40, rot={"base": 1e4, "dims": 8}),
+    "delta_largest_key": delta_layer(1, 1, 512, 16, 2, 8, 8),
     "attention_sizes_of_a_large_model": attention_layer(8, 2, 64, 64, 0.125, window=24, rot={"base": 500000.0, "dims": 64}),
     "feed_forward_beside_attention": attention_layer(1, 1, 8, 8, 1.0, window=2, ff=72),
 }
