@@ -38,7 +38,7 @@ __device__ __forceinline__ float softplus_f32(float x) { return x > 20.f ? x : l
 
 template <typename T, bool FUSE_TAIL>
 __global__ __launch_bounds__(256) void delta_prepare_kernel(
-    const T* __restrict__ proj, int ld, int col_b, const float* __restrict__ a_pre,
+    const T* __restrict__ proj, int ld, int col_b, const float* __restrict__ a_pre, int ld_a,
     const float* __restrict__ conv_w, int taps, const float* __restrict__ a_log,
     const float* __restrict__ dt_bias, float* __restrict__ state, size_t state_stride,
     size_t tail_off, const int* __restrict__ q_start, const int* __restrict__ token_req,
@@ -95,7 +95,7 @@ __global__ __launch_bounds__(256) void delta_prepare_kernel(
     const float rate = expf(a_log[h]);
     for (int i = lane; i < dk; i += TK_WAVE) {
       const int x = h * dk + i;
-      out[decay_off + x] = expf(-rate * softplus_f32(a_pre[(size_t)t * H * dk + x] + dt_bias[x]));
+      out[decay_off + x] = expf(-rate * softplus_f32(a_pre[(size_t)t * ld_a + x] + dt_bias[x]));
     }
   } else {
     for (int i = lane; i < H; i += TK_WAVE)
@@ -321,13 +321,13 @@ __global__ __launch_bounds__(NQ > 2 ? 384 : 1024) void delta_rule_kernel(
 // --------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void gated_head_norm_kernel(const float* __restrict__ o, const float* __restrict__ gate,
-                                                              const float* __restrict__ w, float eps,
+                                                              int ld_gate, int H, const float* __restrict__ w, float eps,
                                                               T* __restrict__ out, long units, int dv) {
   const int lane = threadIdx.x & (TK_WAVE - 1);
   const long unit = (long)blockIdx.x * (blockDim.x / TK_WAVE) + threadIdx.x / TK_WAVE;
   if (unit >= units) return;
   const float* x = o + (size_t)unit * dv;
-  const float* g = gate + (size_t)unit * dv;
+  const float* g = gate + (size_t)(unit / H) * ld_gate + (size_t)(unit % H) * dv;
   float ss = 0.f;
   for (int i = lane; i < dv; i += TK_WAVE) ss = fmaf(x[i], x[i], ss);
   ss = wave_sum(ss);
@@ -336,7 +336,7 @@ __global__ __launch_bounds__(256) void gated_head_norm_kernel(const float* __res
     out[(size_t)unit * dv + i] = from_f32<T>(x[i] * rstd * w[i] * sigmoid_f32(g[i]));
 }
 
-TK_API int tk_delta_prepare(int dt, const void* proj, int ld, int col_b, const float* a_pre,
+TK_API int tk_delta_prepare(int dt, const void* proj, int ld, int col_b, const float* a_pre, int ld_a,
                             const float* conv_w, int taps, const float* a_log, const float* dt_bias,
                             float* state, size_t state_stride, size_t tail_off, const int* q_start,
                             const int* token_req, const int* slots, float* rec, int ld_rec, int n_tokens,
@@ -346,6 +346,7 @@ TK_API int tk_delta_prepare(int dt, const void* proj, int ld, int col_b, const f
   TK_REQUIRE(taps >= 1 && taps <= DR_MAX_TAPS, "delta_prepare: %d taps (1..%d)", taps, DR_MAX_TAPS);
   const int C = 2 * G * dk + H * dv;
   TK_REQUIRE(ld >= C && col_b >= 0 && col_b + H <= ld, "delta_prepare: row stride %d too short", ld);
+  TK_REQUIRE(ld_a >= H * dk, "delta_prepare: the decay projection's stride %d is too short", ld_a);
   TK_REQUIRE(ld_rec >= C + H * dk + H, "delta_prepare: output stride %d too short", ld_rec);
   TK_REQUIRE(tail_off + (size_t)(taps - 1) * C <= state_stride, "delta_prepare: the state row is too short");
   TK_REQUIRE(dk <= DP_MAX_PER_LANE * TK_WAVE && dv <= DP_MAX_PER_LANE * TK_WAVE, "delta_prepare: head sizes %d, %d (at most %d)",
@@ -357,7 +358,7 @@ TK_API int tk_delta_prepare(int dt, const void* proj, int ld, int col_b, const f
   // every request brings one token: the convolving lane moves its channel's tail on itself
   const bool fuse_tail = n_tokens == n_requests && taps > 1;
 #define DP_LAUNCH(T, FUSE)                                                                                         \
-  hipLaunchKernelGGL((delta_prepare_kernel<T, FUSE>), grid, dim3(256), 0, stream, (const T*)proj, ld, col_b, a_pre, \
+  hipLaunchKernelGGL((delta_prepare_kernel<T, FUSE>), grid, dim3(256), 0, stream, (const T*)proj, ld, col_b, a_pre, ld_a, \
                      conv_w, taps, a_log, dt_bias, state, state_stride, tail_off, q_start, token_req, slots, rec,  \
                      ld_rec, H, G, dk, dv)
   if (dt == TK_F32) {
@@ -423,18 +424,19 @@ TK_API int tk_delta_rule(const float* rec, int ld_rec, float* state, size_t stat
   return 0;
 }
 
-TK_API int tk_gated_head_norm(int dt, const float* o, const float* gate, const float* w, float eps, void* out,
+TK_API int tk_gated_head_norm(int dt, const float* o, const float* gate, int ld_gate, const float* w, float eps, void* out,
                               int n_tokens, int H, int dv, hipStream_t stream) {
+  TK_REQUIRE(ld_gate >= H * dv, "gated_head_norm: the gate's stride %d is too short", ld_gate);
   TK_REQUIRE(n_tokens >= 0 && H > 0 && dv > 0, "gated_head_norm: bad sizes %d %d %d", n_tokens, H, dv);
   if (n_tokens == 0) return 0;
   const long units = (long)n_tokens * H;
   const long blocks = (units + 3) / 4;
   TK_REQUIRE(blocks < (1l << 31), "gated_head_norm: too many rows");
   if (dt == TK_F32)
-    hipLaunchKernelGGL(gated_head_norm_kernel<float>, dim3((unsigned)blocks), dim3(256), 0, stream, o, gate, w, eps,
+    hipLaunchKernelGGL(gated_head_norm_kernel<float>, dim3((unsigned)blocks), dim3(256), 0, stream, o, gate, ld_gate, H, w, eps,
                        (float*)out, units, dv);
   else
-    hipLaunchKernelGGL(gated_head_norm_kernel<bf16_t>, dim3((unsigned)blocks), dim3(256), 0, stream, o, gate, w, eps,
+    hipLaunchKernelGGL(gated_head_norm_kernel<bf16_t>, dim3((unsigned)blocks), dim3(256), 0, stream, o, gate, ld_gate, H, w, eps,
                        (bf16_t*)out, units, dv);
   TK_CHECK_LAUNCH("gated_head_norm");
   return 0;

@@ -45,10 +45,10 @@ _SIGNATURES: dict[str, dict[str, list]] = {
         "tk_attention_tile_f32": [c_int, _P, c_int, _P, c_int, _P, _P, _P, c_int, _P, _P, _P, _P] + [c_int] * 7
         + [c_float, _P, c_int, c_int, _P],
         "tk_attention_tile_f32_fits": [c_int] * 5,
-        "tk_delta_prepare": [c_int, _P, c_int, c_int, _P, _P, c_int, _P, _P, _P, c_size_t, c_size_t, _P, _P, _P, _P]
+        "tk_delta_prepare": [c_int, _P, c_int, c_int, _P, c_int, _P, c_int, _P, _P, _P, c_size_t, c_size_t, _P, _P, _P, _P]
         + [c_int] * 7 + [_P],
         "tk_delta_rule": [_P, c_int, _P, c_size_t, _P, _P, _P] + [c_int] * 6 + [_P],
-        "tk_gated_head_norm": [c_int, _P, _P, _P, c_float, _P, c_int, c_int, c_int, _P],
+        "tk_gated_head_norm": [c_int, _P, _P, c_int, _P, c_float, _P, c_int, c_int, c_int, _P],
         "tk_sample": [_P, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P],
         "tk_sample_static": [_P, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P],
         "tk_sample_chunks": [c_int],

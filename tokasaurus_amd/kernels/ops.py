@@ -1299,8 +1299,8 @@ def delta_prepare(
     _need(conv_w.dim() == 2 and conv_w.shape[0] == channels and conv_w.dtype == torch.float32 and conv_w.is_contiguous(),
           f"delta_prepare: the convolutions' weights must be contiguous float32 [{channels}, taps]")
     taps = conv_w.shape[1]
-    _need(a_pre.shape == (n, heads * key_dim) and a_pre.dtype == torch.float32 and a_pre.is_contiguous(),
-          "delta_prepare: the decay's projection must be contiguous float32 [tokens, heads * key_dim]")
+    _need(a_pre.shape == (n, heads * key_dim) and a_pre.dtype == torch.float32 and a_pre.stride(1) == 1,
+          "delta_prepare: the decay's projection must be float32 [tokens, heads * key_dim] with unit inner stride")
     _f32_vector(a_log, heads, "delta_prepare: a_log")
     _f32_vector(dt_bias, heads * key_dim, "delta_prepare: dt_bias")
     _need(state.dim() == 2 and state.dtype == torch.float32 and state.is_contiguous()
@@ -1311,7 +1311,7 @@ def delta_prepare(
     width = delta_rec_width(heads, kv_heads, key_dim, value_dim)
     rec = torch.empty((n, width), dtype=torch.float32, device=proj.device)
     call("tk_delta_prepare", dtype_code(proj.dtype), proj.data_ptr(), proj.stride(0), int(col_b), a_pre.data_ptr(),
-         conv_w.data_ptr(), taps, a_log.data_ptr(), dt_bias.data_ptr(), state.data_ptr(), state.stride(0),
+         a_pre.stride(0) if n > 1 else heads * key_dim, conv_w.data_ptr(), taps, a_log.data_ptr(), dt_bias.data_ptr(), state.data_ptr(), state.stride(0),
          heads * key_dim * value_dim, q_start.data_ptr(), token_req.data_ptr(), slots.data_ptr(), rec.data_ptr(), width,
          n, slots.numel(), heads, kv_heads, key_dim, value_dim, _stream())
     return rec
@@ -1356,10 +1356,11 @@ def gated_head_norm(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, e
     _gpu(o, gate, weight)
     n = o.shape[0]
     for t in (o, gate):
-        _need(t.shape == (n, heads * value_dim) and t.dtype == torch.float32 and t.is_contiguous(),
-              "gated_head_norm: inputs must be contiguous float32 [tokens, heads * value_dim]")
+        _need(t.shape == (n, heads * value_dim) and t.dtype == torch.float32 and t.stride(1) == 1,
+              "gated_head_norm: inputs must be float32 [tokens, heads * value_dim] with unit inner stride")
+    _need(o.is_contiguous(), "gated_head_norm: the recurrence's output must be contiguous")
     _f32_vector(weight, value_dim, "gated_head_norm: the weight")
     out = torch.empty((n, heads * value_dim), dtype=out_dtype, device=o.device)
-    call("tk_gated_head_norm", dtype_code(out_dtype), o.data_ptr(), gate.data_ptr(), weight.data_ptr(), float(eps),
-         out.data_ptr(), n, heads, value_dim, _stream())
+    call("tk_gated_head_norm", dtype_code(out_dtype), o.data_ptr(), gate.data_ptr(), gate.stride(0) if n > 1 else heads * value_dim,
+         weight.data_ptr(), float(eps), out.data_ptr(), n, heads, value_dim, _stream())
     return out

@@ -20,7 +20,7 @@ from __future__ import annotations
 import torch
 
 from tokasaurus_amd.kernels import ops
-from tokasaurus_amd.parts.base import CONV, MIXERS, NORM_WEIGHT, VECTOR, Mixer, StateNeed, StepContext, TensorSpec
+from tokasaurus_amd.parts.base import CONV, MATRIX, MIXERS, NORM_WEIGHT, VECTOR, Mixer, StateNeed, StepContext, TensorSpec
 from tokasaurus_amd.parts.linear import Linear, Placer
 
 
@@ -46,14 +46,17 @@ class ChannelDeltaRule(Mixer):
         self.col_a1 = self.channels
         self.col_g1 = self.col_a1 + self.decay_rank
         self.col_b = self.col_g1 + self.gate_rank
-        self.a2 = Linear(self.decay_rank, [names["a2"]], [num_heads * key_dim])
-        self.g2 = Linear(self.gate_rank, [names["g2"]], [v])
+        # the second halves of the two low-rank projections as one product: the weight is [a2 0; 0 g2], its input
+        # the neighbouring columns a1 | g1 of the stacked product (zeros add nothing to a 32-bit sum)
+        self.low = Linear(self.decay_rank + self.gate_rank, [f"{names['a2']}+{names['g2']}"], [num_heads * key_dim + v])
         self.out = Linear(v, [names["o"]], [hidden_size])
         self.conv_w = self.a_log = self.dt_bias = self.norm_w = None
 
     def tensor_specs(self) -> list[TensorSpec]:
         n, qk, v = self.names, self.num_kv_heads * self.key_dim, self.num_heads * self.value_dim
-        return (self.inp.tensor_specs() + self.a2.tensor_specs() + self.g2.tensor_specs() + self.out.tensor_specs() + [
+        return (self.inp.tensor_specs() + self.out.tensor_specs() + [
+            TensorSpec(n["a2"], (self.num_heads * self.key_dim, self.decay_rank), MATRIX),
+            TensorSpec(n["g2"], (v, self.gate_rank), MATRIX),
             TensorSpec(n["q_conv"], (qk, self.taps), CONV),
             TensorSpec(n["k_conv"], (qk, self.taps), CONV),
             TensorSpec(n["v_conv"], (v, self.taps), CONV),
@@ -67,9 +70,18 @@ class ChannelDeltaRule(Mixer):
                          torch.float32)
 
     def load(self, tensors: dict[str, torch.Tensor], placer: Placer) -> None:
-        for lin in (self.inp, self.a2, self.g2, self.out):
+        for lin in (self.inp, self.out):
             lin.load(tensors, placer)
         n = self.names
+
+        def block_diagonal() -> torch.Tensor:
+            a2, g2 = tensors[n["a2"]], tensors[n["g2"]]
+            w = torch.zeros((a2.shape[0] + g2.shape[0], a2.shape[1] + g2.shape[1]), dtype=placer.dtype)
+            w[: a2.shape[0], : a2.shape[1]] = a2.to(placer.dtype)
+            w[a2.shape[0] :, a2.shape[1] :] = g2.to(placer.dtype)
+            return w.contiguous().to(placer.device)
+
+        self.low.weight = placer.place(("block_diagonal", n["a2"], n["g2"]), block_diagonal)
 
         def f32(key: tuple, make) -> torch.Tensor:
             return placer.place(key, lambda: make().to(torch.float32).contiguous().to(placer.device))
@@ -94,8 +106,8 @@ class ChannelDeltaRule(Mixer):
         assert state is not None, "the delta rule keeps its state in the request's slot"
         H, G, dk, dv = self.num_heads, self.num_kv_heads, self.key_dim, self.value_dim
         proj = self.inp(h)
-        a_pre = self.a2(self._columns(proj, self.col_a1, self.decay_rank), out_f32=True)
-        gate = self.g2(self._columns(proj, self.col_g1, self.gate_rank), out_f32=True)
+        low = self.low(self._columns(proj, self.col_a1, self.decay_rank + self.gate_rank), out_f32=True)
+        a_pre, gate = low[:, : H * dk], low[:, H * dk :]  # 32-bit, rows a stride apart
         rec = ops.delta_prepare(proj, self.col_b, a_pre, self.conv_w, self.a_log, self.dt_bias, state,
                                 ctx.q_start, ctx.token_req, ctx.slots, H, G, dk, dv)
         o = ops.delta_rule(rec, state, ctx.q_start, ctx.slots, H, G, dk, dv)
