@@ -127,11 +127,13 @@ class Prepared:
     """What the product in front of a norm has already done for it, and the norm it did it
     for: either ``data``, the kernels' own record (``kernels.ops.Prenorm``: the rows times
     the norm's weight and partial sums of their squares, which the next product folds in),
-    or ``normed``, the normed rows themselves (made in the pass that added the residual)."""
+    or ``normed``, the normed rows themselves (made in the pass that added the residual; for a
+    block that begins with two norms of the same stream, ``norm`` is its pair of norms and
+    ``normed`` the pair of their rows)."""
 
     data: Any
     norm: "Norm"
-    normed: torch.Tensor | None = None
+    normed: "torch.Tensor | tuple | None" = None
 
 
 @dataclass
