@@ -6,10 +6,34 @@
 //     angle position * freq[i] (32-bit product, 32-bit sine and cosine computed here: no table,
 //     so positions have no upper end),
 //   * writes the queries back in place, the keys and the values into the token's page.
+// Options: query heads of a size `dq` of their own (a query latent normed as one row beside a
+// key latent of another size); `pair_half`: the rotation pairs element i with element
+// i + rot/2 instead of neighbours; `v_from_k`: the row holds no values, a token's values are
+// its keys as they are before the rotation (normed and weighted when the keys are).
 // The arithmetic is 32-bit from the product's rounded output to the one rounding at the store.
-//   row: [nq*dk | nkv*dk | nkv*dv]  (only the first part when !write_cache)
+//   row: [nq*dq | nkv*dk | nkv*dv]  (only the first part when !write_cache; no third part with v_from_k)
 //   K pages: [page][kv head][dk / 8][P][8]    V pages: [page][kv head][P / 4][dv][4]
 #include "common.h"
+
+// The work items of a head of size d of which the leading `rot` elements are rotated: item j names
+// one or two elements (e0, and e1 when `two`) and, when `turned`, the angle they are rotated by.
+struct PairItem {
+  int e0, e1, angle;
+  bool two, turned;
+};
+__device__ __forceinline__ int pair_items(int d, int rot, int pair_half) {
+  return pair_half ? rot / 2 + (d - rot + 1) / 2 : (d + 1) / 2;
+}
+__device__ __forceinline__ PairItem pair_item(int j, int d, int rot, int pair_half) {
+  PairItem it;
+  if (pair_half && j < rot / 2) {
+    it.e0 = j; it.e1 = j + rot / 2; it.angle = j; it.two = true; it.turned = true;
+  } else {
+    const int e = pair_half ? rot + 2 * (j - rot / 2) : 2 * j;
+    it.e0 = e; it.e1 = e + 1; it.angle = e / 2; it.two = e + 1 < d; it.turned = !pair_half && e < rot;
+  }
+  return it;
+}
 
 template <typename T>
 __global__ __launch_bounds__(256) void qk_prepare_kernel(
@@ -17,7 +41,7 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
     const int* __restrict__ token_req, const int* __restrict__ block_table, int table_stride,
     const float* __restrict__ q_weight, const float* __restrict__ k_weight, float eps,
     const float* __restrict__ freq, T* __restrict__ kcache, T* __restrict__ vcache, int nq, int nkv,
-    int dk, int dv, int rot, int P, int write_cache) {
+    int dq, int dk, int dv, int rot, int P, int write_cache, int pair_half, int v_from_k) {
   extern __shared__ float cs[];  // [rot / 2] cosines, [rot / 2] sines
   __shared__ float red[16];
   const int t = blockIdx.x;
@@ -31,7 +55,7 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
     cs[i] = c;
     cs[half + i] = s;
   }
-  const int nqe = nq * dk, nke = nkv * dk;
+  const int nqe = nq * dq, nke = nkv * dk;
   float rq = 1.f, rk = 1.f;
   if (q_weight) {
     float ss = 0.f;
@@ -51,19 +75,19 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
   }
   __syncthreads();  // the table of this token's angles is written
 
-  // queries, in place, a pair of neighbours a thread (a head of odd size ends in a single element)
-  const int hp = (dk + 1) / 2;
-  for (int i = threadIdx.x; i < nq * hp; i += blockDim.x) {
-    const int e = 2 * (i % hp), x = (i / hp) * dk + e;
-    const bool two = e + 1 < dk;
-    float u = to_f32<T>(row[x]) * rq, v = two ? to_f32<T>(row[x + 1]) * rq : 0.f;
+  // queries, in place, a pair a thread (a head of odd size ends in a single element)
+  const int hq = pair_items(dq, rot, pair_half);
+  for (int i = threadIdx.x; i < nq * hq; i += blockDim.x) {
+    const PairItem it = pair_item(i % hq, dq, rot, pair_half);
+    const int x0 = (i / hq) * dq + it.e0, x1 = (i / hq) * dq + it.e1;
+    float u = to_f32<T>(row[x0]) * rq, v = it.two ? to_f32<T>(row[x1]) * rq : 0.f;
     if (q_weight) {
-      u *= q_weight[x];
-      if (two) v *= q_weight[x + 1];
+      u *= q_weight[x0];
+      if (it.two) v *= q_weight[x1];
     }
-    if (e < rot) rotate_pair(u, v, cs[e / 2], cs[half + e / 2], u, v);
-    row[x] = from_f32<T>(u);
-    if (two) row[x + 1] = from_f32<T>(v);
+    if (it.turned) rotate_pair(u, v, cs[it.angle], cs[half + it.angle], u, v);
+    row[x0] = from_f32<T>(u);
+    if (it.two) row[x1] = from_f32<T>(v);
   }
   if (!write_cache) return;
 
@@ -71,19 +95,27 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
   const int p = pos % P;
   const T* krow = row + nqe;
   const T* vrow = krow + nke;
-  for (int i = threadIdx.x; i < nkv * hp; i += blockDim.x) {
-    const int h = i / hp, e = 2 * (i % hp), x = h * dk + e;
-    const bool two = e + 1 < dk;
-    float u = to_f32<T>(krow[x]) * rk, v = two ? to_f32<T>(krow[x + 1]) * rk : 0.f;
+  const int hk = pair_items(dk, rot, pair_half);
+  for (int i = threadIdx.x; i < nkv * hk; i += blockDim.x) {
+    const int h = i / hk;
+    const PairItem it = pair_item(i % hk, dk, rot, pair_half);
+    const int x0 = h * dk + it.e0, x1 = h * dk + it.e1;
+    float u = to_f32<T>(krow[x0]) * rk, v = it.two ? to_f32<T>(krow[x1]) * rk : 0.f;
     if (k_weight) {
-      u *= k_weight[x];
-      if (two) v *= k_weight[x + 1];
+      u *= k_weight[x0];
+      if (it.two) v *= k_weight[x1];
     }
-    if (e < rot) rotate_pair(u, v, cs[e / 2], cs[half + e / 2], u, v);
+    if (v_from_k) {  // the values are the keys as they are here, before the rotation
+      T* vdst = vcache + ((size_t)page * nkv + h) * P * dv;
+      vdst[value_offset(dv, p, it.e0)] = from_f32<T>(u);
+      if (it.two) vdst[value_offset(dv, p, it.e1)] = from_f32<T>(v);
+    }
+    if (it.turned) rotate_pair(u, v, cs[it.angle], cs[half + it.angle], u, v);
     T* dst = kcache + ((size_t)page * nkv + h) * key_page_elems(P, dk);
-    dst[key_offset(P, p, e)] = from_f32<T>(u);
-    if (two) dst[key_offset(P, p, e + 1)] = from_f32<T>(v);
+    dst[key_offset(P, p, it.e0)] = from_f32<T>(u);
+    if (it.two) dst[key_offset(P, p, it.e1)] = from_f32<T>(v);
   }
+  if (v_from_k) return;
   for (int i = threadIdx.x; i < nkv * dv; i += blockDim.x) {
     const int h = i / dv, e = i % dv;
     vcache[((size_t)page * nkv + h) * P * dv + value_offset(dv, p, e)] = vrow[i];
@@ -93,13 +125,14 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
 TK_API int tk_qk_prepare(int dt, void* qkv, int row_stride, const int* positions, const int* token_req,
                          const int* block_table, int table_stride, const float* q_weight,
                          const float* k_weight, float eps, const float* freq, void* kcache, void* vcache,
-                         int n_tokens, int nq, int nkv, int dk, int dv, int rot, int P, int write_cache,
-                         hipStream_t stream) {
-  TK_REQUIRE(n_tokens >= 0 && nq > 0 && nkv >= 0 && dk > 0 && dv > 0 && P > 0,
-             "qk_prepare: bad sizes tokens=%d nq=%d nkv=%d dk=%d dv=%d P=%d", n_tokens, nq, nkv, dk, dv, P);
-  TK_REQUIRE(rot >= 0 && rot <= dk && rot % 2 == 0, "qk_prepare: %d rotated elements of a head of %d", rot, dk);
+                         int n_tokens, int nq, int nkv, int dq, int dk, int dv, int rot, int P, int write_cache,
+                         int pair_half, int v_from_k, hipStream_t stream) {
+  TK_REQUIRE(n_tokens >= 0 && nq > 0 && nkv >= 0 && dq > 0 && dk > 0 && dv > 0 && P > 0,
+             "qk_prepare: bad sizes tokens=%d nq=%d nkv=%d dq=%d dk=%d dv=%d P=%d", n_tokens, nq, nkv, dq, dk, dv, P);
+  TK_REQUIRE(rot >= 0 && rot <= dk && rot <= dq && rot % 2 == 0, "qk_prepare: %d rotated elements of heads of %d and %d", rot, dq, dk);
   TK_REQUIRE(rot == 0 || freq, "qk_prepare: a rotation needs its frequencies");
-  TK_REQUIRE(row_stride >= (write_cache ? nq * dk + nkv * (dk + dv) : nq * dk),
+  TK_REQUIRE(!v_from_k || dv == dk, "qk_prepare: values that are the keys have the keys' size, not %d for %d", dv, dk);
+  TK_REQUIRE(row_stride >= (write_cache ? nq * dq + nkv * (dk + (v_from_k ? 0 : dv)) : nq * dq),
              "qk_prepare: row stride %d is shorter than the heads it holds", row_stride);
   TK_REQUIRE(!write_cache || (kcache && vcache && block_table && nkv > 0), "qk_prepare: cache pointers missing");
   if (n_tokens == 0) return 0;
@@ -107,11 +140,11 @@ TK_API int tk_qk_prepare(int dt, void* qkv, int row_stride, const int* positions
   if (dt == TK_F32)
     hipLaunchKernelGGL(qk_prepare_kernel<float>, dim3(n_tokens), dim3(256), smem, stream, (float*)qkv,
                        row_stride, positions, token_req, block_table, table_stride, q_weight, k_weight, eps,
-                       freq, (float*)kcache, (float*)vcache, nq, nkv, dk, dv, rot, P, write_cache);
+                       freq, (float*)kcache, (float*)vcache, nq, nkv, dq, dk, dv, rot, P, write_cache, pair_half, v_from_k);
   else
     hipLaunchKernelGGL(qk_prepare_kernel<bf16_t>, dim3(n_tokens), dim3(256), smem, stream, (bf16_t*)qkv,
                        row_stride, positions, token_req, block_table, table_stride, q_weight, k_weight, eps,
-                       freq, (bf16_t*)kcache, (bf16_t*)vcache, nq, nkv, dk, dv, rot, P, write_cache);
+                       freq, (bf16_t*)kcache, (bf16_t*)vcache, nq, nkv, dq, dk, dv, rot, P, write_cache, pair_half, v_from_k);
   TK_CHECK_LAUNCH("qk_prepare");
   return 0;
 }

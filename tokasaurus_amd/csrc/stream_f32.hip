@@ -160,6 +160,128 @@ TK_API int tk_residual_norm(int dt, const float* x, const float* a, const float*
 }
 
 // --------------------------------------------------------------------------
+// The update of a stream whose branches are normed before they are added (a norm in front of and
+// behind every sublayer), one row a workgroup:
+//     x_out = x + a / sqrt(mean(a^2) + eps_b) * wb
+// and, when w is given, the row of the norm that reads the new stream,
+//     h = x_out / sqrt(mean(x_out^2) + eps) * w     rounded once to T.
+// x, a, wb, w are 32-bit.  x_out may be x itself.  The row is held in registers between the
+// passes when the width allows (multiples of 4 up to 4 * 256 * RN_QUADS), else read back.
+// --------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void post_norm_residual_kernel(
+    const float* x, const float* __restrict__ a, const float* __restrict__ wb, float eps_b,
+    float* x_out, const float* __restrict__ w, float eps, T* __restrict__ h, int hidden) {
+  __shared__ float red[16];
+  const size_t row = (size_t)blockIdx.x * hidden;
+  float sa = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    const float y = a[row + i];
+    sa = fmaf(y, y, sa);
+  }
+  const float rb = 1.0f / sqrtf(block_sum(sa, red) / (float)hidden + eps_b);
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    const float v = x[row + i] + a[row + i] * rb * wb[i];
+    x_out[row + i] = v;
+    ss = fmaf(v, v, ss);
+  }
+  if (!w) return;
+  const float rstd = 1.0f / sqrtf(block_sum(ss, red) / (float)hidden + eps);
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x)  // a thread reads back what it wrote
+    h[row + i] = from_f32<T>(x_out[row + i] * rstd * w[i]);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void post_norm_residual_vec_kernel(
+    const float* x, const float* __restrict__ a, const float* __restrict__ wb, float eps_b,
+    float* x_out, const float* __restrict__ w, float eps, T* __restrict__ h, int hidden) {
+  __shared__ float red[16];
+  const size_t row = (size_t)blockIdx.x * hidden;
+  const int quads = hidden / 4;
+  float4 v[RN_QUADS];
+  float sa = 0.f;
+#pragma unroll
+  for (int j = 0; j < RN_QUADS; ++j) {
+    const int i = threadIdx.x + j * 256;
+    if (i < quads) {
+      v[j] = ((const float4*)(a + row))[i];
+      sa = fmaf(v[j].x, v[j].x, sa); sa = fmaf(v[j].y, v[j].y, sa);
+      sa = fmaf(v[j].z, v[j].z, sa); sa = fmaf(v[j].w, v[j].w, sa);
+    }
+  }
+  const float rb = 1.0f / sqrtf(block_sum(sa, red) / (float)hidden + eps_b);
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < RN_QUADS; ++j) {
+    const int i = threadIdx.x + j * 256;
+    if (i < quads) {
+      const float4 xv = ((const float4*)(x + row))[i];
+      const float4 g = ((const float4*)wb)[i];
+      v[j].x = xv.x + v[j].x * rb * g.x; v[j].y = xv.y + v[j].y * rb * g.y;
+      v[j].z = xv.z + v[j].z * rb * g.z; v[j].w = xv.w + v[j].w * rb * g.w;
+      ((float4*)(x_out + row))[i] = v[j];
+      ss = fmaf(v[j].x, v[j].x, ss); ss = fmaf(v[j].y, v[j].y, ss);
+      ss = fmaf(v[j].z, v[j].z, ss); ss = fmaf(v[j].w, v[j].w, ss);
+    }
+  }
+  if (!w) return;
+  const float rstd = 1.0f / sqrtf(block_sum(ss, red) / (float)hidden + eps);
+#pragma unroll
+  for (int j = 0; j < RN_QUADS; ++j) {
+    const int i = threadIdx.x + j * 256;
+    if (i < quads) {
+      const float4 g = ((const float4*)w)[i];
+      const float n[4] = {v[j].x * rstd * g.x, v[j].y * rstd * g.y, v[j].z * rstd * g.z, v[j].w * rstd * g.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) h[row + 4 * i + e] = from_f32<T>(n[e]);
+    }
+  }
+}
+
+TK_API int tk_post_norm_residual(int dt, const float* x, const float* a, const float* wb, float eps_b, float* x_out,
+                                 const float* w, float eps, void* h, int rows, int hidden, hipStream_t stream) {
+  TK_REQUIRE(rows >= 0 && hidden > 0, "post_norm_residual: bad sizes %d %d", rows, hidden);
+  TK_REQUIRE(x && a && wb && x_out && (!w || h), "post_norm_residual: a pointer is missing");
+  if (rows == 0) return 0;
+  const uintptr_t all = (uintptr_t)x | (uintptr_t)a | (uintptr_t)wb | (uintptr_t)x_out | (uintptr_t)w;
+  const bool vec = hidden % 4 == 0 && hidden <= 4 * 256 * RN_QUADS && (all & 15) == 0;
+#define PNR_LAUNCH(K, T) hipLaunchKernelGGL(K<T>, dim3(rows), dim3(256), 0, stream, x, a, wb, eps_b, x_out, w, eps, (T*)h, hidden)
+  if (vec) {
+    if (dt == TK_F32) PNR_LAUNCH(post_norm_residual_vec_kernel, float); else PNR_LAUNCH(post_norm_residual_vec_kernel, bf16_t);
+  } else {
+    if (dt == TK_F32) PNR_LAUNCH(post_norm_residual_kernel, float); else PNR_LAUNCH(post_norm_residual_kernel, bf16_t);
+  }
+#undef PNR_LAUNCH
+  TK_CHECK_LAUNCH("post_norm_residual");
+  return 0;
+}
+
+// --------------------------------------------------------------------------
+// out[t, :] = T([x[t, :] | y[t, :]]): two 32-bit streams side by side, rounded once to the storage
+// type that a product reads.
+// --------------------------------------------------------------------------
+template <typename T>
+__global__ void concat_cast_kernel(const float* __restrict__ x, const float* __restrict__ y, T* __restrict__ out, int hidden) {
+  const size_t row = blockIdx.x;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    out[row * 2 * hidden + i] = from_f32<T>(x[row * hidden + i]);
+    out[row * 2 * hidden + hidden + i] = from_f32<T>(y[row * hidden + i]);
+  }
+}
+
+TK_API int tk_concat_cast(int dt, const float* x, const float* y, void* out, int rows, int hidden, hipStream_t stream) {
+  TK_REQUIRE(rows >= 0 && hidden > 0 && x && y && out, "concat_cast: bad arguments");
+  if (rows == 0) return 0;
+  if (dt == TK_F32)
+    hipLaunchKernelGGL(concat_cast_kernel<float>, dim3(rows), dim3(256), 0, stream, x, y, (float*)out, hidden);
+  else
+    hipLaunchKernelGGL(concat_cast_kernel<bf16_t>, dim3(rows), dim3(256), 0, stream, x, y, (bf16_t*)out, hidden);
+  TK_CHECK_LAUNCH("concat_cast");
+  return 0;
+}
+
+// --------------------------------------------------------------------------
 // logits <- cap * tanh(logits / cap), in place, 32-bit.
 // --------------------------------------------------------------------------
 __global__ void softcap_kernel(float* __restrict__ v, size_t n, float cap) {

@@ -41,7 +41,14 @@ _SIGNATURES: dict[str, dict[str, list]] = {
         "tk_embed_scaled": [c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_float, _P],
         "tk_residual_norm": [c_int, _P, _P, _P, c_float, _P, _P, _P, c_float, c_float, _P, _P, c_int, c_int, _P],
         "tk_softcap": [_P, c_size_t, c_float, _P],
-        "tk_qk_prepare": [c_int, _P, c_int, _P, _P, _P, c_int, _P, _P, c_float, _P, _P, _P] + [c_int] * 8 + [_P],
+        "tk_qk_prepare": [c_int, _P, c_int, _P, _P, _P, c_int, _P, _P, c_float, _P, _P, _P] + [c_int] * 11 + [_P],
+        "tk_post_norm_residual": [c_int, _P, _P, _P, c_float, _P, _P, c_float, _P, c_int, c_int, _P],
+        "tk_concat_cast": [c_int, _P, _P, _P, c_int, c_int, _P],
+        "tk_expert_route": [c_int, _P, c_int, _P, _P, _P] + [c_int] * 6 + [_P, _P, _P, _P],
+        "tk_expert_gate_up": [c_int, _P, c_int, _P, _P, _P] + [c_int] * 5 + [_P],
+        "tk_expert_combine": [c_int, _P, c_int, _P, _P, _P, _P, _P, _P, _P] + [c_int] * 5 + [_P],
+        "tk_head_linear": [c_int, _P, c_int, _P, _P, c_int, c_int] + [c_int] * 4 + [_P],
+        "tk_squared_relu": [c_int, _P, c_size_t, _P],
         "tk_attention_tile_f32": [c_int, _P, c_int, _P, c_int, _P, _P, _P, c_int, _P, _P, _P, _P] + [c_int] * 7
         + [c_float, _P, c_int, c_int, _P],
         "tk_attention_tile_f32_fits": [c_int] * 5,

@@ -1170,24 +1170,33 @@ def qk_prepare(
     value_dim: int,
     page_size: int,
     write_cache: bool = True,
+    query_dim: int | None = None,
+    pair_halves: bool = False,
+    values_are_keys: bool = False,
 ) -> None:
-    """In place on the rows [q: nq*dk | k: nkv*dk | v: nkv*dv] (only q when not ``write_cache``):
+    """In place on the rows [q: nq*dq | k: nkv*dk | v: nkv*dv] (only q when not ``write_cache``):
     the RMS norm of the whole query row and of the whole key row (32-bit weights of those sizes,
     or None for no norm), the rotation of elements (2i, 2i+1) of every head by position *
-    freq[i] for i < len(freq), and the append of keys and values to the token's page."""
+    freq[i] for i < len(freq), and the append of keys and values to the token's page.
+    ``query_dim``: the size dq of a query head where it is not a key head's.  ``pair_halves``:
+    the rotation pairs element i with element i + len(freq) instead of neighbours.
+    ``values_are_keys``: the rows hold no values; a token's values are its keys as they are
+    before the rotation (after the norm, when there is one)."""
     _gpu(qkv, positions, token_req, block_table, q_weight, k_weight, freq, kcache, vcache)
     _need(qkv.dim() == 2 and qkv.stride(1) == 1, "qk_prepare: rows must be 2-d with unit inner stride")
     n = qkv.shape[0]
-    need = nq * key_dim + (nkv * (key_dim + value_dim) if write_cache else 0)
+    dq = key_dim if query_dim is None else int(query_dim)
+    _need(not values_are_keys or value_dim == key_dim, "qk_prepare: values that are the keys have the keys' size")
+    need = nq * dq + (nkv * (key_dim + (0 if values_are_keys else value_dim)) if write_cache else 0)
     _need(qkv.shape[1] >= need, f"qk_prepare: rows of {qkv.shape[1]} hold no {need} elements")
     _i32(positions, "positions")
     _i32(token_req, "token_req")
     _need(positions.numel() == n and token_req.numel() == n, "positions/token_req must have one entry a token")
-    _f32_vector(q_weight, nq * key_dim, "qk_prepare: the query norm's weight")
+    _f32_vector(q_weight, nq * dq, "qk_prepare: the query norm's weight")
     _f32_vector(k_weight, nkv * key_dim, "qk_prepare: the key norm's weight")
     rot = 0
     if freq is not None:
-        _need(freq.dim() == 1 and freq.dtype == torch.float32 and freq.is_contiguous() and 2 * freq.numel() <= key_dim,
+        _need(freq.dim() == 1 and freq.dtype == torch.float32 and freq.is_contiguous() and 2 * freq.numel() <= min(key_dim, dq),
               "qk_prepare: frequencies must be contiguous float32, at most half a head's size of them")
         rot = 2 * freq.numel()
     if write_cache:
@@ -1199,7 +1208,8 @@ def qk_prepare(
          q_weight.data_ptr() if q_weight is not None else None, k_weight.data_ptr() if k_weight is not None else None,
          float(eps), freq.data_ptr() if freq is not None else None,
          kcache.data_ptr() if write_cache else None, vcache.data_ptr() if write_cache else None,
-         n, nq, nkv if write_cache else 0, key_dim, value_dim, rot, page_size, 1 if write_cache else 0, _stream())
+         n, nq, nkv if write_cache else 0, dq, key_dim, value_dim, rot, page_size, 1 if write_cache else 0,
+         1 if pair_halves else 0, 1 if values_are_keys else 0, _stream())
 
 
 def attention_tile_f32_fits(nq: int, nkv: int, key_dim: int, value_dim: int, page_size: int) -> bool:
@@ -1363,4 +1373,126 @@ def gated_head_norm(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, e
     out = torch.empty((n, heads * value_dim), dtype=out_dtype, device=o.device)
     call("tk_gated_head_norm", dtype_code(out_dtype), o.data_ptr(), gate.data_ptr(), gate.stride(0) if n > 1 else heads * value_dim,
          weight.data_ptr(), float(eps), out.data_ptr(), n, heads, value_dim, _stream())
+    return out
+
+
+# --------------------------------------------------------------------------
+# a stream whose branches are normed before they are added
+# --------------------------------------------------------------------------
+
+def post_norm_residual(x: torch.Tensor, branch: torch.Tensor, branch_weight: torch.Tensor, branch_eps: float,
+                       weight: torch.Tensor | None = None, eps: float = 0.0, out_dtype: torch.dtype = torch.float32,
+                       in_place: bool = True) -> tuple[torch.Tensor, torch.Tensor | None]:
+    """``x_new = x + branch / sqrt(mean(branch^2) + branch_eps) * branch_weight`` on a 32-bit
+    stream (the branch 32-bit too), and, when ``weight`` is given, the rows of the norm that
+    reads the new stream, ``x_new / sqrt(mean(x_new^2) + eps) * weight`` rounded once to
+    ``out_dtype``.  Returns (x_new, those rows or None).  ``in_place``: x_new overwrites x."""
+    _gpu(x, branch, branch_weight, weight)
+    _need(x.dim() == 2 and x.dtype == torch.float32 and x.is_contiguous(), "post_norm_residual: the stream must be contiguous float32 [rows, H]")
+    _need(branch.shape == x.shape and branch.dtype == torch.float32 and branch.is_contiguous(),
+          "post_norm_residual: the branch must be contiguous float32 of the stream's shape")
+    rows, hidden = x.shape
+    _f32_vector(branch_weight, hidden, "post_norm_residual: the branch norm's weight")
+    _f32_vector(weight, hidden, "post_norm_residual: a norm weight")
+    x_out = x if in_place else torch.empty_like(x)
+    h = torch.empty((rows, hidden), dtype=out_dtype, device=x.device) if weight is not None else None
+    if rows:
+        call("tk_post_norm_residual", dtype_code(out_dtype), x.data_ptr(), branch.data_ptr(), branch_weight.data_ptr(),
+             float(branch_eps), x_out.data_ptr(), weight.data_ptr() if weight is not None else None, float(eps),
+             h.data_ptr() if h is not None else None, rows, hidden, _stream())
+    return x_out, h
+
+
+def concat_cast(x: torch.Tensor, y: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """[x | y] row by row for two 32-bit streams of one shape, rounded once to ``out_dtype``."""
+    _gpu(x, y)
+    _need(x.dim() == 2 and x.dtype == torch.float32 and x.is_contiguous() and y.shape == x.shape and y.dtype == torch.float32
+          and y.is_contiguous(), "concat_cast: two contiguous float32 streams of one shape")
+    out = torch.empty((x.shape[0], 2 * x.shape[1]), dtype=out_dtype, device=x.device)
+    if x.shape[0]:
+        call("tk_concat_cast", dtype_code(out_dtype), x.data_ptr(), y.data_ptr(), out.data_ptr(), x.shape[0], x.shape[1], _stream())
+    return out
+
+
+def squared_relu_(x: torch.Tensor) -> torch.Tensor:
+    """x <- max(x, 0)^2, in place."""
+    _gpu(x)
+    _need(x.is_contiguous(), "squared_relu: the rows must be contiguous")
+    call("tk_squared_relu", dtype_code(x.dtype), x.data_ptr(), x.numel(), _stream())
+    return x
+
+
+# --------------------------------------------------------------------------
+# a matrix a head; experts of which a token uses a few
+# --------------------------------------------------------------------------
+
+def head_linear(x: torch.Tensor, w: torch.Tensor, out_f32: bool = False) -> torch.Tensor:
+    """y[t, h, :] = w[h] x[t, h, :] for w [heads, out, in] and the leading heads * in columns of
+    the rows of x; returns [tokens, heads * out] in x's type, or 32-bit sums with ``out_f32``."""
+    _gpu(x, w)
+    _need(w.dim() == 3 and w.is_contiguous() and w.dtype == x.dtype, "head_linear: weights contiguous [heads, out, in] of the rows' type")
+    heads, n_out, n_in = w.shape
+    _need(x.dim() == 2 and x.stride(1) == 1 and x.shape[1] >= heads * n_in, "head_linear: rows of unit inner stride that hold heads * in columns")
+    y = torch.empty((x.shape[0], heads * n_out), dtype=torch.float32 if out_f32 else x.dtype, device=x.device)
+    if x.shape[0]:
+        call("tk_head_linear", dtype_code(x.dtype), x.data_ptr(), x.stride(0), w.data_ptr(), y.data_ptr(), y.stride(0),
+             1 if (out_f32 and x.dtype != torch.float32) else 0, x.shape[0], heads, n_in, n_out, _stream())
+    return y
+
+
+def expert_route(h: torch.Tensor, w_router: torch.Tensor, correction: torch.Tensor, groups: int, keep: int, top: int,
+                 w_gate: torch.Tensor | None = None) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor | None]:
+    """The router of a mixture of experts, 32-bit arithmetic: logits ``w_router h`` over all
+    experts, their softmax s, the choice by ``s + correction`` among the experts of the ``keep``
+    groups of neighbours (of ``groups`` equal ones) whose best choice score is largest, ties to the
+    left.  Returns ids [tokens, top] int32 in the order of the choice scores, weights [tokens, top]
+    (the chosen experts' s), and, with ``w_gate`` [width], sigmoid(w_gate . h) [tokens]."""
+    _gpu(h, w_router, correction, w_gate)
+    n_all, width = w_router.shape
+    _need(h.dim() == 2 and h.stride(1) == 1 and h.shape[1] == width and w_router.dtype == h.dtype and w_router.is_contiguous(),
+          "expert_route: rows [tokens, width] and a contiguous router [experts, width] of one type")
+    _f32_vector(correction, n_all, "expert_route: the correction")
+    _need(w_gate is None or (w_gate.numel() == width and w_gate.dtype == h.dtype and w_gate.is_contiguous()),
+          "expert_route: the shared expert's gate must be contiguous [width]")
+    n = h.shape[0]
+    ids = torch.empty((n, top), dtype=torch.int32, device=h.device)
+    weights = torch.empty((n, top), dtype=torch.float32, device=h.device)
+    gate = torch.empty((n,), dtype=torch.float32, device=h.device) if w_gate is not None else None
+    if n == 0:
+        return ids, weights, gate
+    call("tk_expert_route", dtype_code(h.dtype), h.data_ptr(), h.stride(0), w_router.data_ptr(), correction.data_ptr(),
+         w_gate.data_ptr() if w_gate is not None else None, n, width, n_all, int(groups), int(keep), int(top),
+         ids.data_ptr(), weights.data_ptr(), gate.data_ptr() if gate is not None else None, _stream())
+    return ids, weights, gate
+
+
+def expert_mix(h: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor,
+               shared: torch.Tensor | None = None, shared_gate: torch.Tensor | None = None) -> torch.Tensor:
+    """The weighted sum of a token's chosen experts, 32-bit [tokens, width]: expert e is
+    ``w_down[e] (silu(gate) * up)`` with [gate | up] = ``w_gate_up[e] h``; an id from
+    ``len(w_down)`` on names an identity expert (its output is h), a negative id an empty
+    place.  ``shared`` (32-bit [tokens, width]) times ``shared_gate`` [tokens] is added."""
+    _gpu(h, w_gate_up, w_down, ids, weights, shared, shared_gate)
+    experts, two_ff, width = w_gate_up.shape
+    ff = two_ff // 2
+    _need(w_gate_up.is_contiguous() and w_down.is_contiguous() and w_down.shape == (experts, width, ff)
+          and w_gate_up.dtype == h.dtype and w_down.dtype == h.dtype, "expert_mix: weights [experts, 2 ff, width] and [experts, width, ff] of the rows' type")
+    _need(h.dim() == 2 and h.stride(1) == 1 and h.shape[1] == width, "expert_mix: rows [tokens, width]")
+    n = h.shape[0]
+    _i32(ids, "ids")
+    top = ids.shape[1]
+    _need(ids.shape == (n, top) and weights.shape == (n, top) and weights.dtype == torch.float32 and weights.is_contiguous(),
+          "expert_mix: ids and weights [tokens, top]")
+    if shared is not None:
+        _need(shared.shape == (n, width) and shared.dtype == torch.float32 and shared.is_contiguous(), "expert_mix: the shared expert's rows must be float32 [tokens, width]")
+        _f32_vector(shared_gate, n, "expert_mix: the shared expert's gate")
+    out = torch.empty((n, width), dtype=torch.float32, device=h.device)
+    if n == 0:
+        return out
+    inter = torch.empty((n * top, ff), dtype=h.dtype, device=h.device)
+    call("tk_expert_gate_up", dtype_code(h.dtype), h.data_ptr(), h.stride(0), w_gate_up.data_ptr(), ids.data_ptr(),
+         inter.data_ptr(), n, width, ff, experts, top, _stream())
+    call("tk_expert_combine", dtype_code(h.dtype), h.data_ptr(), h.stride(0), inter.data_ptr(), w_down.data_ptr(),
+         ids.data_ptr(), weights.data_ptr(), shared.data_ptr() if shared is not None else None,
+         shared_gate.data_ptr() if shared is not None else None, out.data_ptr(), n, width, ff, experts, top, _stream())
     return out

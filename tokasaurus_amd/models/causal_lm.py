@@ -8,7 +8,7 @@ import torch
 
 from tokasaurus_amd.kernels import ops
 from tokasaurus_amd.models.spec import ModelSpec
-from tokasaurus_amd.parts.base import (BLOCKS, EMBEDDINGS, HEADS, CacheNeed, CacheView, Part, Prepared, StateNeed, StepContext,
+from tokasaurus_amd.parts.base import (BLOCKS, CONNECTORS, EMBEDDINGS, HEADS, CacheNeed, CacheView, Part, Prepared, StateNeed, StepContext,
                                        TensorSpec)
 from tokasaurus_amd.parts.block import build_with_shared, stream_and_prepared
 import tokasaurus_amd.parts.embedding  # noqa: F401  (registers the embedding and the head)
@@ -27,13 +27,14 @@ class CausalLM:
         self.embedding = build_with_shared(EMBEDDINGS, spec.embedding, self.shared)
         self.blocks = [build_with_shared(BLOCKS, b, self.shared) for b in spec.layers]
         self.head = build_with_shared(HEADS, spec.head, self.shared)
+        self.connectors = [build_with_shared(CONNECTORS, c, self.shared) for c in spec.connectors]
         self.dtype: torch.dtype | None = None
         self.device: torch.device | None = None
         self.weight_bytes = 0
 
     # ---- tensors
     def parts(self) -> list[Part]:
-        return [self.embedding, *self.blocks, self.head]
+        return [self.embedding, *self.connectors, *self.blocks, self.head]
 
     def tensor_specs(self) -> list[TensorSpec]:
         seen: dict[str, TensorSpec] = {}
@@ -75,11 +76,17 @@ class CausalLM:
         order = self.spec.run_order
         last = len(order) - 1
         prepared = None  # what a block has done for the norm that the next one (or the head) starts with
+        # a connector reads the embedding's output again; blocks may update the stream in place
+        x0 = x.clone() if self.connectors else None
         for i, entry in enumerate(order):
             rows = want_rows if i == last else None
             block = self.blocks[entry.layer]
+            if entry.before is not None:
+                x, prepared = self.connectors[entry.before].forward(x, x0), None
             if block.fuses_norm:
                 next_norm = self.blocks[order[i + 1].layer].entry_norm() if i < last else self.head.entry_norm()
+                if i < last and order[i + 1].before is not None:
+                    next_norm = None  # the stream changes before the next block reads it
                 out = block.forward(x, ctx, caches[i], states[i], rows, prepared=prepared, next_norm=next_norm)
             else:
                 out = block.forward(x, ctx, caches[i], states[i], rows)

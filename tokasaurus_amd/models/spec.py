@@ -3,7 +3,8 @@ layers run.
 
 ``run_order`` is a list of entries; an entry names a layer (the same layer may
 be named twice: its weights are then used twice, each use with a cache of its
-own) and may name an earlier entry whose cache it reads instead of keeping one.
+own) and may name an earlier entry whose cache it reads instead of keeping one, and a
+connector that runs on the stream right before it.
 """
 
 from __future__ import annotations
@@ -17,6 +18,7 @@ from tokasaurus_amd.parts.base import PartSpec
 class RunEntry:
     layer: int
     cache_of: int | None = None  # index into run_order of the entry whose cache is read
+    before: int | None = None  # index into ModelSpec.connectors of what runs on the stream right before this entry
 
 
 @dataclass(frozen=True)
@@ -31,9 +33,13 @@ class ModelSpec:
     # tensors a checkpoint of this architecture may carry although the model reads them from
     # elsewhere (the head's matrix of a checkpoint that ties it to the embedding)
     ignorable_tensors: tuple[str, ...] = ()
+    # what happens to the stream between blocks (chosen from parts.base.CONNECTORS), named by run entries
+    connectors: tuple[PartSpec, ...] = ()
 
     def validate(self) -> None:
         for i, e in enumerate(self.run_order):
+            if e.before is not None and not 0 <= e.before < len(self.connectors):
+                raise ValueError(f"run entry {i} names connector {e.before}, the model has {len(self.connectors)}")
             if not 0 <= e.layer < len(self.layers):
                 raise ValueError(f"run entry {i} names layer {e.layer}, the model has {len(self.layers)}")
             if e.cache_of is not None:

@@ -27,6 +27,7 @@ NORM_WEIGHT = "norm_weight"  # a norm's scale vector: 1 + N(0, 0.01) when random
 NORM_OFFSET = "norm_offset"  # a norm's scale stored around zero (the norm multiplies by 1 + w): N(0, 0.01) when random
 VECTOR = "vector"  # a learned vector of another role (a sink, a rate, a step's bias): N(0, 0.5) when random
 CONV = "conv"  # the taps of short convolutions, [channels, taps]: N(0, 0.5) when random
+SMALL_VECTOR = "small_vector"  # a learned vector that nudges (a router's correction): N(0, 0.01) when random
 INT_TABLE = "int_table"  # integer table: kept as int32
 
 
@@ -280,6 +281,16 @@ class Head(Part):
         raise NotImplementedError
 
 
+class Connector(Part):
+    """What a model does to its residual stream between two blocks, outside any block: it gets
+    the stream ``x`` and the embedding's output ``x0`` of the same rows and returns the new
+    stream (a new tensor: ``x0`` is read again later).  A run entry names the connector that
+    runs before it (``models.spec.RunEntry.before``)."""
+
+    def forward(self, x: torch.Tensor, x0: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+
 class Block(Part):
     """The arrangement of norms, a mixer and a feed-forward around the residual stream.
 
@@ -365,5 +376,6 @@ POSITION_ENCODINGS = Registry("position encoding")
 MIXERS = Registry("mixer")
 FEED_FORWARDS = Registry("feed-forward")
 BLOCKS = Registry("block arrangement")
+CONNECTORS = Registry("connector")
 EMBEDDINGS = Registry("embedding")
 HEADS = Registry("head")

@@ -15,11 +15,13 @@ import torch
 from tokasaurus_amd.kernels import ops
 from tokasaurus_amd.parts.base import (
     BLOCKS,
+    CONNECTORS,
     FEED_FORWARDS,
     MIXERS,
     NORMS,
     Block,
     CacheView,
+    Connector,
     Normed,
     Part,
     Prepared,
@@ -27,7 +29,7 @@ from tokasaurus_amd.parts.base import (
     StepContext,
     TensorSpec,
 )
-from tokasaurus_amd.parts.linear import Placer
+from tokasaurus_amd.parts.linear import Linear, Placer
 
 
 def build_with_shared(registry, spec: PartSpec, shared: dict):
@@ -184,3 +186,95 @@ class ParallelResidualBlock(Block):
         if first is None:
             return x
         return x, Prepared(None, next_norm, (g1, g2) if isinstance(next_norm, NormPair) else g1)
+
+
+@BLOCKS.register("sandwich_norm")
+class SandwichNormBlock(Block):
+    """A norm in front of and behind every sublayer, on a 32-bit residual stream:
+        x <- x + post1(mixer(norm1(x)));  x <- x + post2(ff(norm2(x)))
+    ``feed_forward`` (with its two norms) may be absent.  The branches hand over their last
+    products' 32-bit sums; one kernel norms a branch, adds it to the stream and writes the rows
+    of the norm that reads the new stream (this block's second, the next block's first, or the
+    head's).  The norms are ``stream_rmsnorm``s; the mixer must have ``mix`` and the
+    feed-forward ``transform``."""
+
+    fuses_norm = True
+
+    def __init__(self, mixer_norm: PartSpec, mixer: PartSpec, mixer_post_norm: PartSpec, ff_norm: PartSpec | None = None,
+                 feed_forward: PartSpec | None = None, ff_post_norm: PartSpec | None = None, shared: dict | None = None):
+        shared = shared if shared is not None else {}
+        if len({ff_norm is None, feed_forward is None, ff_post_norm is None}) != 1:
+            raise ValueError("a feed-forward and its two norms come together")
+        self.mixer_norm = build_with_shared(NORMS, mixer_norm, shared)
+        self.mixer = build_with_shared(MIXERS, mixer, shared)
+        self.mixer_post_norm = build_with_shared(NORMS, mixer_post_norm, shared)
+        self.ff_norm = build_with_shared(NORMS, ff_norm, shared) if ff_norm is not None else None
+        self.feed_forward = build_with_shared(FEED_FORWARDS, feed_forward, shared) if feed_forward is not None else None
+        self.ff_post_norm = build_with_shared(NORMS, ff_post_norm, shared) if ff_post_norm is not None else None
+        for n in (self.mixer_norm, self.mixer_post_norm, self.ff_norm, self.ff_post_norm):
+            if n is not None and (getattr(n, "same_rule", None) is None or n.unit_offset):
+                raise ValueError("a sandwich_norm block takes stream_rmsnorm norms with plain weights")
+
+    def children(self) -> list[Part]:
+        return [c for c in (self.mixer_norm, self.mixer, self.mixer_post_norm, self.ff_norm, self.feed_forward, self.ff_post_norm)
+                if c is not None]
+
+    def tensor_specs(self) -> list[TensorSpec]:
+        return [s for c in self.children() for s in c.tensor_specs()]
+
+    def load(self, tensors: dict[str, torch.Tensor], placer: Placer) -> None:
+        for c in self.children():
+            c.load(tensors, placer)
+
+    def entry_norm(self):
+        return self.mixer_norm
+
+    @staticmethod
+    def _add(x, branch, post, reader):
+        """Norm the branch, add it, and write the rows of ``reader`` (a plain-weight stream norm or None)."""
+        ok = reader is not None and getattr(reader, "same_rule", None) is not None and not reader.unit_offset
+        return ops.post_norm_residual(x, branch, post.weight, post.eps, reader.weight if ok else None,
+                                      reader.eps if ok else 0.0, reader.out_dtype if ok else torch.float32)
+
+    def forward(self, x, ctx: StepContext, cache, state, rows, prepared: Prepared | None = None, next_norm=None):
+        if x.dtype != torch.float32:
+            raise TypeError("a sandwich_norm block runs on a 32-bit stream (an embedding with stream_f32)")
+        if prepared is not None and prepared.norm is self.mixer_norm and prepared.normed is not None:
+            h = prepared.normed
+        else:
+            h = self.mixer_norm.forward(x)
+        a = self.mixer.mix(h, ctx, cache, state, rows, out_f32=True)
+        if rows is not None:
+            x = ops.gather_rows(x, rows)
+        tap = ctx.extras.get("stream_tap")
+        reader = self.ff_norm if self.feed_forward is not None else next_norm
+        x, h = self._add(x, a, self.mixer_post_norm, reader)
+        if self.feed_forward is not None:
+            b = self.feed_forward.transform(h, out_f32=True)
+            reader = next_norm
+            x, h = self._add(x, b, self.ff_post_norm, reader)
+        if tap is not None:  # a list that collects the stream after every block (tests, debugging)
+            tap.append(x.clone())
+        if h is None:
+            return x
+        return x, Prepared(None, reader, h)
+
+
+@CONNECTORS.register("embedding_mix")
+class EmbeddingMix(Connector):
+    """x <- W [x; x0]: the stream and the embedding's output side by side through one matrix
+    [width, 2 width] (the stream's columns first).  Both are 32-bit streams; they are rounded
+    once to the storage type for the product, whose 32-bit sums are the new stream."""
+
+    def __init__(self, hidden_size: int, name: str):
+        self.hidden_size = hidden_size
+        self.proj = Linear(2 * hidden_size, [name], [hidden_size])
+
+    def tensor_specs(self) -> list[TensorSpec]:
+        return self.proj.tensor_specs()
+
+    def load(self, tensors: dict[str, torch.Tensor], placer: Placer) -> None:
+        self.proj.load(tensors, placer)
+
+    def forward(self, x: torch.Tensor, x0: torch.Tensor) -> torch.Tensor:
+        return self.proj(ops.concat_cast(x, x0, self.proj.weight.dtype), out_f32=True)

@@ -1,10 +1,12 @@
 """Dense gated feed-forward (tokasaurus/model/llama.py:290-339):
-``x + down(silu(gate(h)) * up(h))``, no biases.  gate and up are one stacked product."""
+``x + down(silu(gate(h)) * up(h))``, no biases.  gate and up are one stacked product.
+Beside it the ungated feed-forward whose activation is the square of relu."""
 
 from __future__ import annotations
 
 import torch
 
+from tokasaurus_amd.kernels import ops
 from tokasaurus_amd.parts.base import FEED_FORWARDS, FeedForward, Normed, TensorSpec
 from tokasaurus_amd.parts.linear import Linear, Placer
 
@@ -33,3 +35,27 @@ class SwiGLU(FeedForward):
         """The feed-forward's own output, nothing added: for blocks that combine their branches
         themselves.  ``out_f32``: the down projection's 32-bit sums leave unrounded."""
         return self.down(self.gate_up(h, swiglu=True), out_f32=out_f32)
+
+
+@FEED_FORWARDS.register("squared_relu")
+class SquaredReLU(FeedForward):
+    """``down(max(up(h), 0)^2)``, no gate and no biases."""
+
+    def __init__(self, hidden_size: int, intermediate_size: int, names: dict[str, str]):
+        self.hidden_size = hidden_size
+        self.intermediate_size = intermediate_size
+        self.up = Linear(hidden_size, [names["up"]], [intermediate_size])
+        self.down = Linear(intermediate_size, [names["down"]], [hidden_size])
+
+    def tensor_specs(self) -> list[TensorSpec]:
+        return self.up.tensor_specs() + self.down.tensor_specs()
+
+    def load(self, tensors: dict[str, torch.Tensor], placer: Placer) -> None:
+        self.up.load(tensors, placer)
+        self.down.load(tensors, placer)
+
+    def forward(self, h: torch.Tensor, residual: torch.Tensor):
+        return self.down(ops.squared_relu_(self.up(h)), residual=residual)
+
+    def transform(self, h: torch.Tensor, out_f32: bool = False) -> torch.Tensor:
+        return self.down(ops.squared_relu_(self.up(h)), out_f32=out_f32)

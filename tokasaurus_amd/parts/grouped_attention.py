@@ -2,9 +2,11 @@
 not have, each a parameter: key and value heads of different sizes, a scale of the model's
 choosing, RMS norms of the queries and of the keys over the whole projection (all heads at
 once), a rotation of neighbouring elements of the leading part of a head, a sliding window, a
-learned sink per query head in the softmax's denominator, and keys and values taken from
-another layer's cache (the run entry's ``cache_of``; the mixer then has no key and value
-tensors).
+learned sink per query head in the softmax's denominator (or one constant score for all heads),
+keys and values taken from another layer's cache (the run entry's ``cache_of``; the mixer then
+has no key and value tensors), a rotation that pairs the two halves of a head's leading part
+instead of neighbours, and values that are the keys themselves as projected, before the rotation
+(the mixer then has no value tensor).
 
 Scores, softmax weights, norms, angles and the rotation are 32-bit arithmetic in either storage
 type.  One kernel norms, rotates and appends (``ops.qk_prepare``); the attention itself runs on
@@ -71,13 +73,17 @@ class GroupedAttention(Mixer):
         sink_name: str | None = None,
         own_kv: bool = True,
         shared: dict | None = None,
+        sink_value: float | None = None,
+        values_are_keys: bool = False,
     ):
         """``names``: checkpoint names of the q, k, v, o matrices (k and v only with ``own_kv``).
         ``projection_norm``: ``{"q": name, "k": name, "eps": eps}``, weights of the whole
         projections' sizes (k only with ``own_kv``).  ``window``: a query sees itself and the
         window - 1 positions before it (0: all).  ``cache_window``: how far back the cache keeps
         keys (0: all): at least ``window``, more when another layer reads this cache further
-        back; by default ``window``.  ``sink_name``: one number a query head."""
+        back; by default ``window``.  ``sink_name``: one number a query head.  ``sink_value``: no
+        tensor, every head's sink has this score (0: one is added to the softmax's denominator).
+        ``values_are_keys``: ``names`` has no v; a token's values are its keys before the rotation."""
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads are not a multiple of {num_kv_heads} kv heads")
         self.hidden_size, self.num_heads, self.num_kv_heads = hidden_size, num_heads, num_kv_heads
@@ -90,8 +96,16 @@ class GroupedAttention(Mixer):
         self.own_kv = bool(own_kv)
         self.projection_norm = dict(projection_norm) if projection_norm else None
         self.sink_name = sink_name
-        sizes = [num_heads * key_dim] + ([num_kv_heads * key_dim, num_kv_heads * value_dim] if own_kv else [])
-        self.qkv = Linear(hidden_size, [names["q"]] + ([names["k"], names["v"]] if own_kv else []), sizes)
+        self.sink_value = None if sink_value is None else float(sink_value)
+        if sink_name and sink_value is not None:
+            raise ValueError("a sink is learned (sink_name) or constant (sink_value), not both")
+        self.values_are_keys = bool(values_are_keys)
+        if self.values_are_keys and (self.value_dim != self.key_dim or not own_kv):
+            raise ValueError("values that are the keys have the keys' size and come with keys of the mixer's own")
+        kv_sizes = [num_kv_heads * key_dim] + ([] if self.values_are_keys else [num_kv_heads * value_dim])
+        kv_names = [names["k"]] + ([] if self.values_are_keys else [names["v"]])
+        sizes = [num_heads * key_dim] + (kv_sizes if own_kv else [])
+        self.qkv = Linear(hidden_size, [names["q"]] + (kv_names if own_kv else []), sizes)
         self.out = Linear(num_heads * value_dim, [names["o"]], [hidden_size])
         self.q_norm_weight: torch.Tensor | None = None
         self.k_norm_weight: torch.Tensor | None = None
@@ -135,6 +149,9 @@ class GroupedAttention(Mixer):
                 self.k_norm_weight = f32(self.projection_norm["k"])
         if self.sink_name:
             self.sink = f32(self.sink_name)
+        elif self.sink_value is not None:
+            self.sink = placer.place(("constant_f32", self.sink_value, self.num_heads), lambda: torch.full(
+                (self.num_heads,), self.sink_value, dtype=torch.float32, device=placer.device))
         if self.position is not None:
             self.position.prepare(placer.device)
 
@@ -148,7 +165,9 @@ class GroupedAttention(Mixer):
         ops.qk_prepare(qkv, ctx.positions, ctx.token_req, cache.block_table, self.q_norm_weight,
                        self.k_norm_weight if self.own_kv else None, eps,
                        self.position.freq if self.position is not None else None,
-                       cache.keys, cache.values, nq, nkv, dk, dv, cache.page_size, write_cache=self.own_kv)
+                       cache.keys, cache.values, nq, nkv, dk, dv, cache.page_size, write_cache=self.own_kv,
+                       pair_halves=self.position is not None and self.position.pair_halves,
+                       values_are_keys=self.values_are_keys)
         if ops.attention_tile_f32_fits(nq, nkv, dk, dv, cache.page_size):
             gg = ops.attention_tile_heads(nq // nkv, ctx.max_q_len)
             tile_req, tile_row0 = tile_plan(ctx, 16 // gg)

@@ -1,0 +1,108 @@
+"""Attention whose keys and values are expanded, head by head, from one small latent a token, and
+only that latent is cached.
+
+Per token: the query latent ``cq = norm(W_dq h)`` and the key/value latent ``c = norm(W_dkv h)``
+(RMS norms with weights, 32-bit); ``q = W_uq cq``; per head ``k = W_uk c`` and ``v = W_uv c``;
+``score = (q . k) * scale`` over every earlier token and the token itself, an ordinary softmax,
+no positions; the output projection reads the heads side by side.
+
+The engine never expands a cached token's keys or values.  Since ``q_h . (W_uk,h c) =
+(W_uk,h^T q_h) . c`` and ``sum_j p_j W_uv,h c_j = W_uv,h sum_j p_j c_j``, a head's query is taken
+into the latent's space (a matrix a head, ``ops.head_linear``), the attention runs with ONE
+key/value head whose keys and values are both the latent (every query head reads it: the
+arithmetic intensity of the cache is that of ``num_heads`` queries a key), and the head's
+result is taken from the latent's space to its values by ``W_uv,h``.  The pages hold the
+latent twice, once in the key layout and once in the value layout, ``2 * kv_rank`` numbers a
+token and layer where expanded keys and values would take ``num_heads * (key_dim + value_dim)``.
+
+Scores, softmax weights and norms are 32-bit arithmetic in either storage type; the kernels are
+those of ``grouped_attention`` (``ops.qk_prepare`` norms both latents and appends,
+``ops.attention_tile_f32`` or, for sizes it does not take, ``ops.paged_attention_generic``).
+"""
+
+from __future__ import annotations
+
+import torch
+
+from tokasaurus_amd.kernels import ops
+from tokasaurus_amd.parts.base import MATRIX, MIXERS, NORM_WEIGHT, CacheNeed, CacheView, Mixer, StepContext, TensorSpec
+from tokasaurus_amd.parts.grouped_attention import tile_plan
+from tokasaurus_amd.parts.linear import Linear, Placer
+
+
+@MIXERS.register("latent_attention")
+class LatentAttention(Mixer):
+    def __init__(self, hidden_size: int, num_heads: int, key_dim: int, value_dim: int, q_rank: int, kv_rank: int, scale: float,
+                 norm_eps: float, names: dict[str, str]):
+        """``names``: checkpoint names under the keys dq, dkv ([rank, hidden]), dq_norm, dkv_norm
+        ([rank]), uq ([heads * key_dim, q_rank]), uk ([heads * key_dim, kv_rank]), uv
+        ([heads * value_dim, kv_rank]), o ([hidden, heads * value_dim])."""
+        self.hidden_size, self.num_heads = hidden_size, num_heads
+        self.key_dim, self.value_dim, self.q_rank, self.kv_rank = int(key_dim), int(value_dim), int(q_rank), int(kv_rank)
+        self.scale, self.norm_eps = float(scale), float(norm_eps)
+        self.names = dict(names)
+        self.down = Linear(hidden_size, [names["dq"], names["dkv"]], [self.q_rank, self.kv_rank])
+        self.up_q = Linear(self.q_rank, [names["uq"]], [num_heads * self.key_dim])
+        self.out = Linear(num_heads * self.value_dim, [names["o"]], [hidden_size])
+        self.q_norm_weight = self.c_norm_weight = None
+        self.to_latent: torch.Tensor | None = None  # [heads, kv_rank, key_dim]: W_uk,h transposed
+        self.from_latent: torch.Tensor | None = None  # [heads, value_dim, kv_rank]: W_uv,h
+
+    def tensor_specs(self) -> list[TensorSpec]:
+        n, H = self.names, self.num_heads
+        return self.down.tensor_specs() + self.up_q.tensor_specs() + self.out.tensor_specs() + [
+            TensorSpec(n["dq_norm"], (self.q_rank,), NORM_WEIGHT),
+            TensorSpec(n["dkv_norm"], (self.kv_rank,), NORM_WEIGHT),
+            TensorSpec(n["uk"], (H * self.key_dim, self.kv_rank), MATRIX),
+            TensorSpec(n["uv"], (H * self.value_dim, self.kv_rank), MATRIX),
+        ]
+
+    def cache_need(self) -> CacheNeed:
+        return CacheNeed(1, self.kv_rank, 0, 0)
+
+    def check_cache(self, page_size: int, dtype: torch.dtype) -> None:
+        ops.check_attention_shape(dtype, self.num_heads, 1, self.kv_rank, page_size, value_dim=self.kv_rank, generic_only=True)
+
+    def load(self, tensors: dict[str, torch.Tensor], placer: Placer) -> None:
+        for lin in (self.down, self.up_q, self.out):
+            lin.load(tensors, placer)
+        n, H = self.names, self.num_heads
+
+        def f32(name: str) -> torch.Tensor:
+            return placer.place(("vector_f32", name), lambda: tensors[name].to(torch.float32).contiguous().to(placer.device))
+
+        self.q_norm_weight, self.c_norm_weight = f32(n["dq_norm"]), f32(n["dkv_norm"])
+        self.to_latent = placer.place(("heads_transposed", n["uk"]), lambda: tensors[n["uk"]].to(placer.dtype).view(
+            H, self.key_dim, self.kv_rank).transpose(1, 2).contiguous().to(placer.device))
+        self.from_latent = placer.place(("heads", n["uv"]), lambda: tensors[n["uv"]].to(placer.dtype).view(
+            H, self.value_dim, self.kv_rank).contiguous().to(placer.device))
+
+    def _attend(self, h: torch.Tensor, ctx: StepContext, cache: CacheView, rows: torch.Tensor | None) -> torch.Tensor:
+        assert cache is not None and cache.writable, "latent attention keeps its latent in a cache of its own"
+        H, r = self.num_heads, self.kv_rank
+        lat = self.down(h)  # [cq | c]
+        # both latents normed (each over its whole length), the key/value latent appended as key and as value
+        ops.qk_prepare(lat, ctx.positions, ctx.token_req, cache.block_table, self.q_norm_weight, self.c_norm_weight,
+                       self.norm_eps, None, cache.keys, cache.values, 1, 1, r, r, cache.page_size,
+                       query_dim=self.q_rank, values_are_keys=True)
+        cq = lat[:, : self.q_rank]
+        if lat.dtype != torch.float32 and (self.q_rank % 8 or lat.stride(0) % 8):
+            cq = torch.empty((lat.shape[0], self.q_rank), dtype=lat.dtype, device=lat.device).copy_(cq)
+        q = ops.head_linear(self.up_q(cq), self.to_latent)  # [tokens, heads * kv_rank]
+        if ops.attention_tile_f32_fits(H, 1, r, r, cache.page_size):
+            gg = ops.attention_tile_heads(H, ctx.max_q_len)
+            tile_req, tile_row0 = tile_plan(ctx, 16 // gg)
+            o = ops.attention_tile_f32(q, cache.keys, cache.values, cache.block_table, ctx.q_start, ctx.kv_len,
+                                       tile_req, tile_row0, H, 1, r, r, cache.page_size, gg, scale=self.scale)
+        else:
+            o = ops.paged_attention_generic(q, cache.keys, cache.values, cache.block_table, ctx.token_req, ctx.positions,
+                                            H, 1, r, cache.page_size, scale=self.scale, value_dim=r)
+        if rows is not None:
+            o = ops.gather_rows(o, rows)
+        return ops.head_linear(o, self.from_latent)  # [tokens, heads * value_dim]
+
+    def mix(self, h, ctx, cache, state, rows, out_f32: bool = False):
+        return self.out(self._attend(h, ctx, cache, rows), out_f32=out_f32)
+
+    def forward(self, h, residual, ctx, cache, state, rows):
+        return self.out(self._attend(h, ctx, cache, rows), residual=residual)

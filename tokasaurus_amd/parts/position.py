@@ -93,6 +93,8 @@ class InterleavedRotary(PositionEncoding):
     by the angle position * f_i.  It keeps the frequencies only: the kernel that rotates
     multiplies and takes sine and cosine in 32-bit itself, so positions have no upper end."""
 
+    pair_halves = False  # which elements form a pair: neighbours (2i, 2i+1), or (i, i + dims/2)
+
     def __init__(self, dims: int, base: float, scaling: dict | None = None):
         if dims % 2 or dims <= 0:
             raise ValueError(f"a rotation of pairs needs an even number of elements, got {dims}")
@@ -104,3 +106,11 @@ class InterleavedRotary(PositionEncoding):
     def prepare(self, device: torch.device) -> None:
         if self.freq is None:
             self.freq = interleaved_frequencies(self.dims, self.base, self.scaling).to(device)
+
+
+@POSITION_ENCODINGS.register("rotary_halves")
+class HalvesRotary(InterleavedRotary):
+    """The same angles, position * f_i with f_i = base^(-2i/dims), for the pairs (i, i + dims/2) of
+    the leading ``dims`` elements of a head; computed in the kernel like its parent's."""
+
+    pair_halves = True

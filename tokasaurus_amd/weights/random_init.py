@@ -3,7 +3,7 @@ configuration and a seed.  The reference has no such mode (it only fabricates
 inputs, tokasaurus/manager/input_building.py:14-100).
 
 Every matrix is drawn from N(0, 0.02), every norm weight from 1 + N(0, 0.01) (from N(0, 0.01)
-when it is stored around zero), other learned vectors from N(0, 0.5),
+when it is stored around zero, as is a vector that only nudges), other learned vectors from N(0, 0.5),
 in 32-bit on the host, in the sorted order of the tensor names, from one
 generator seeded with ``seed``; integer tables are drawn uniformly.  Tensors are
 stored in bfloat16, so the 32-bit engine, the bfloat16 engine and any plain
@@ -20,7 +20,7 @@ import torch
 from safetensors.torch import save_file
 
 from tokasaurus_amd.models.registry import architecture_of
-from tokasaurus_amd.parts.base import BIAS, CONV, INT_TABLE, MATRIX, NORM_OFFSET, NORM_WEIGHT, VECTOR, TensorSpec
+from tokasaurus_amd.parts.base import BIAS, CONV, INT_TABLE, MATRIX, NORM_OFFSET, NORM_WEIGHT, SMALL_VECTOR, VECTOR, TensorSpec
 
 MATRIX_STD = 0.02
 NORM_STD = 0.01
@@ -44,7 +44,7 @@ def draw_tensors(
             t = torch.randn(spec.shape, generator=gen, dtype=torch.float32, device=device) * MATRIX_STD
         elif spec.kind == NORM_WEIGHT:
             t = 1.0 + torch.randn(spec.shape, generator=gen, dtype=torch.float32, device=device) * NORM_STD
-        elif spec.kind == NORM_OFFSET:
+        elif spec.kind in (NORM_OFFSET, SMALL_VECTOR):
             t = torch.randn(spec.shape, generator=gen, dtype=torch.float32, device=device) * NORM_STD
         elif spec.kind in (VECTOR, CONV):
             t = torch.randn(spec.shape, generator=gen, dtype=torch.float32, device=device) * VECTOR_STD
