@@ -82,7 +82,7 @@ def parse() -> argparse.Namespace:
                    help="instead of the decode steps, a case that shapes of one length do not show (prints its own line): "
                         "chunked-prefill: one prompt of --context tokens in portions of --portion tokens; "
                         "mixed-decode: decode steps of --batch - 1 requests of --short tokens beside one of --context tokens")
-    p.add_argument("--design", default=None, choices=["kupuzen"],
+    p.add_argument("--design", default=None, choices=["kupuzen", "taborax"],
                    help="instead of the decode steps: prefill and decode of this design at layer sizes of --design-sizes "
                         "beside the Llama shape of equal width, heads, feed-forward and layers (prints its own line)")
     p.add_argument("--design-sizes", default="1b,3b", help="which sizes of DESIGN_SIZES, comma separated")
@@ -360,6 +360,32 @@ def kupuzen_like(size: dict, layers: int) -> dict:
             "layers": [attention if i % 4 == 3 else delta for i in range(layers)]}
 
 
+# A Taborax of the same width, vocabulary and number of layer runs: latent attention (the Llama heads over a latent of
+# 256) and, every third layer, grouped attention whose values are its keys (the Llama heads, half of each rotated);
+# the first layer's feed-forward is dense with the Llama inner size, the others are mixtures whose six chosen experts
+# and shared expert together have that inner size (32 experts and 2 identity experts in 4 groups, 2 kept); two inner
+# layers are passed twice, so `layers` layer runs use `layers - 2` layers' weights.
+def taborax_like(size: dict, layers: int) -> dict:
+    ll = size["llama"]
+    d = ll["hidden_size"] // ll["num_attention_heads"]
+    inner = ll["intermediate_size"]
+    mixture = {"kind": "moe", "expert": {"ff": inner // 8}, "shared": {"ff": inner // 4},
+               "router": {"experts": 32, "identity": 2, "top": 6, "groups": {"count": 2, "keep": 1}}}
+    latent = {"type": "latent_attention", "mixer": {"heads": ll["num_attention_heads"], "dim": d, "vdim": d, "q_rank": 512,
+                                                    "kv_rank": 256, "scale": d ** -0.5}}
+    attention = {"type": "attention", "mixer": {
+        "heads": ll["num_attention_heads"], "kv_heads": ll["num_key_value_heads"], "dim": d, "vdim": d, "scale": d ** -0.5,
+        "rot": {"base": ll["rope_theta"], "dims": d // 2}}}
+    distinct = max(layers - 2, 3)
+    made = []
+    for i in range(distinct):
+        layer = dict(attention if i % 3 == 2 else latent)
+        layer["mlp"] = {"kind": "dense", "ff": inner} if i == 0 else mixture
+        made.append(layer)
+    return {"architecture": "Taborax", "vocab": ll["vocab_size"], "width": ll["hidden_size"], "norm": {"eps": 1e-6},
+            "loop": {"start": 1, "stop": 3, "times": 2}, "layers": made}
+
+
 def run_design(args) -> int:
     """Prefill of one prompt and decode steps of the new design beside the Llama shape of equal
     size, both with seeded random weights through the same runner and engine."""
@@ -372,7 +398,7 @@ def run_design(args) -> int:
     for name in [x for x in args.design_sizes.split(",") if x]:
         size = DESIGN_SIZES[name]
         configs = {"llama": dict(size["llama"], num_hidden_layers=args.design_layers),
-                   args.design: kupuzen_like(size, args.design_layers)}
+                   args.design: (kupuzen_like if args.design == "kupuzen" else taborax_like)(size, args.design_layers)}
         if args.design_only:
             del configs["llama"]
         rec = {}

@@ -41,7 +41,7 @@ __global__ __launch_bounds__(NW * TK_WAVE) void attention_tile_f32_kernel(
     const int* __restrict__ q_start, const int* __restrict__ kv_len, const int* __restrict__ tile_req,
     const int* __restrict__ tile_row0, int nq, int nkv, int dk, int dv, int P, int window, float scale,
     const float* __restrict__ sink, int gg) {
-  extern __shared__ float merge[];  // SPLIT: [waves][16] maxima, [waves][16] sums, [waves][VT][4][64] weighted values
+  extern __shared__ float merge[];  // SPLIT: [waves][16] maxima, [waves][16] sums, [waves - 1][VT][4][64] weighted values
   const int lane = threadIdx.x & (TK_WAVE - 1), wave = threadIdx.x / TK_WAVE;
   const int group = nq / nkv;
   const int blocks_per_kv = group / gg;  // head blocks of gg heads
@@ -219,10 +219,13 @@ __global__ __launch_bounds__(NW * TK_WAVE) void attention_tile_f32_kernel(
       sm[wave * 16 + col] = m_run;
       sl[wave * 16 + col] = l;
     }
+    // (the first wavefront adds the others' sums to its own, which never leave its registers)
+    if (wave > 0) {
 #pragma unroll
-    for (int t = 0; t < VT; ++t)
+      for (int t = 0; t < VT; ++t)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) so[((wave * VT + t) * 4 + i) * TK_WAVE + lane] = o[t][i];
+        for (int i = 0; i < 4; ++i) so[(((wave - 1) * VT + t) * 4 + i) * TK_WAVE + lane] = o[t][i];
+    }
     __syncthreads();
     if (wave != 0) return;
     float m_all = -INFINITY;
@@ -230,16 +233,19 @@ __global__ __launch_bounds__(NW * TK_WAVE) void attention_tile_f32_kernel(
     for (int w = 0; w < NW; ++w) m_all = fmaxf(m_all, sm[w * 16 + col]);
     l = 0.f;
 #pragma unroll
-    for (int t = 0; t < VT; ++t) o[t] = (v4f){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
     for (int w = 0; w < NW; ++w) {
       const float mw = sm[w * 16 + col];
       const float f = (mw == -INFINITY) ? 0.f : expf(mw - m_all);
       l = fmaf(sl[w * 16 + col], f, l);
+      if (w == 0) {
 #pragma unroll
-      for (int t = 0; t < VT; ++t)
+        for (int t = 0; t < VT; ++t) o[t] = o[t] * f;
+      } else {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) o[t][i] = fmaf(so[((w * VT + t) * 4 + i) * TK_WAVE + lane], f, o[t][i]);
+        for (int t = 0; t < VT; ++t)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) o[t][i] = fmaf(so[(((w - 1) * VT + t) * 4 + i) * TK_WAVE + lane], f, o[t][i]);
+      }
     }
     m_run = m_all;
   }
@@ -276,7 +282,7 @@ static void at_launch(dim3 grid, bool split, hipStream_t stream, const void* q, 
   if (split) {
     // eight wavefronts a tile where their sums fit the local memory, else four
     constexpr int NW = VT <= 4 ? 8 : 4;
-    const size_t smem = sizeof(float) * NW * (32 + (size_t)VT * 4 * TK_WAVE);
+    const size_t smem = sizeof(float) * (NW * 32 + (size_t)(NW - 1) * VT * 4 * TK_WAVE);
     hipLaunchKernelGGL((attention_tile_f32_kernel<T, KM, VT, true, NW>), grid, dim3(NW * TK_WAVE), smem, stream,
                        (const T*)q, q_stride, (T*)out, out_stride, (const T*)kcache, (const T*)vcache, block_table,
                        table_stride, q_start, kv_len, tile_req, tile_row0, nq, nkv, dk, dv, P, window, scale, sink, gg);
@@ -302,7 +308,7 @@ TK_API int tk_attention_tile_f32(int dt, const void* q, int q_stride, void* out,
   if (n_tiles <= 0) return 0;
   const int head_blocks = nkv * (group / gg);
   const int km = (dk + 31) / 32, vt = dv / 16;
-  const bool sp = split && vt <= 8;  // the sums of a wider value head do not fit the local memory
+  const bool sp = split != 0;
   const dim3 grid(n_tiles, sp ? head_blocks : (head_blocks + AT_WAVES - 1) / AT_WAVES);
   TK_REQUIRE(grid.y < 65536, "attention_tile_f32: too many heads");
 #define AT_ARGS grid, sp, stream, q, q_stride, out, out_stride, kcache, vcache, block_table, table_stride, q_start, kv_len, \

@@ -29,7 +29,7 @@ IN_TREE_DIR = Path(__file__).resolve().parent / "_build"
 GROUPS = {
     "core": ["errors.hip", "elementwise.hip", "attention_generic.hip", "gemm_generic.hip", "sample.hip", "step_io.hip",
              "stream_f32.hip", "attention_prepare.hip", "attention_tile_f32.hip", "delta_rule.hip", "routed_experts.hip"],
-    "mfma": ["errors.hip", "attention_mfma.hip", "gemm_mfma.hip"],
+    "mfma": ["errors.hip", "attention_mfma.hip", "gemm_mfma.hip", "grouped_gemm.hip"],
     "library": ["errors.hip", "gemm_library.hip"],
 }
 # what a group's library is linked with beside the HIP runtime

@@ -69,6 +69,10 @@ _SIGNATURES: dict[str, dict[str, list]] = {
         + [c_float, c_int, c_int, c_int, c_int, _P, _P, _P, c_int, _P],
         "tk_gemm_skinny_bf16": [_P, c_int, _P, _P, c_int, _P, c_int, _P] + [c_int] * 9 + [_P],
         "tk_gemm_skinny_parts": [c_int, c_int, c_int],
+        "tk_grouped_gemm_bf16": [_P, c_int, _P, _P, _P, c_int, c_int, c_int, c_int, _P, c_size_t, _P, c_int, c_int, c_int, c_int,
+                                 c_int, c_int, _P],
+        "tk_expert_sort": [_P, c_int, c_int, c_int, c_int, _P, _P, _P, _P],
+        "tk_expert_sum": [_P, c_int, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, _P],
     },
     "library": {
         "tk_gemm_library_bf16": [_P, c_int, _P, c_int, _P, c_int, c_int, c_int, c_int, c_int, _P, c_size_t, _P],

@@ -1426,6 +1426,17 @@ def squared_relu_(x: torch.Tensor) -> torch.Tensor:
 # a matrix a head; experts of which a token uses a few
 # --------------------------------------------------------------------------
 
+GROUPED_TILE = 32  # slots a tile of the grouped matrix-core product (GG_TM of grouped_gemm.hip)
+GROUPED_FROM_ROWS = 16  # rows above which the products of experts and of heads run in tiles on the matrix cores
+
+
+def _grouped_takes(x: torch.Tensor, w: torch.Tensor, inner: int) -> bool:
+    """Whether the grouped matrix-core product takes these rows and weights: bfloat16, rows that start at
+    multiples of 16 bytes."""
+    return (x.dtype == torch.bfloat16 and inner % 8 == 0 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
+            and w.data_ptr() % 16 == 0)
+
+
 def head_linear(x: torch.Tensor, w: torch.Tensor, out_f32: bool = False) -> torch.Tensor:
     """y[t, h, :] = w[h] x[t, h, :] for w [heads, out, in] and the leading heads * in columns of
     the rows of x; returns [tokens, heads * out] in x's type, or 32-bit sums with ``out_f32``."""
@@ -1434,6 +1445,12 @@ def head_linear(x: torch.Tensor, w: torch.Tensor, out_f32: bool = False) -> torc
     heads, n_out, n_in = w.shape
     _need(x.dim() == 2 and x.stride(1) == 1 and x.shape[1] >= heads * n_in, "head_linear: rows of unit inner stride that hold heads * in columns")
     y = torch.empty((x.shape[0], heads * n_out), dtype=torch.float32 if out_f32 else x.dtype, device=x.device)
+    if x.shape[0] > GROUPED_FROM_ROWS and _grouped_takes(x, w, n_in):
+        # many rows: tiles of 32 rows on the matrix cores, the head as the tile's group
+        tiles = -(-x.shape[0] // GROUPED_TILE)
+        call("tk_grouped_gemm_bf16", x.data_ptr(), x.stride(0), None, None, None, tiles, heads, n_in, n_out, w.data_ptr(),
+             n_out * n_in, y.data_ptr(), y.stride(0), n_out, n_in, x.shape[0], 0, 1 if out_f32 else 0, _stream())
+        return y
     if x.shape[0]:
         call("tk_head_linear", dtype_code(x.dtype), x.data_ptr(), x.stride(0), w.data_ptr(), y.data_ptr(), y.stride(0),
              1 if (out_f32 and x.dtype != torch.float32) else 0, x.shape[0], heads, n_in, n_out, _stream())
@@ -1488,6 +1505,24 @@ def expert_mix(h: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor, i
         _f32_vector(shared_gate, n, "expert_mix: the shared expert's gate")
     out = torch.empty((n, width), dtype=torch.float32, device=h.device)
     if n == 0:
+        return out
+    if n > GROUPED_FROM_ROWS and _grouped_takes(h, w_gate_up, width) and ff % 8 == 0 and w_down.data_ptr() % 16 == 0:
+        # many tokens: the pairs sorted by expert, every expert's rows in tiles on the matrix cores
+        max_tiles = -(-(n * top) // GROUPED_TILE) + experts
+        slots = max_tiles * GROUPED_TILE
+        book = torch.empty((2 * slots + max_tiles,), dtype=torch.int32, device=h.device)
+        slot_pair, slot_token, tile_group = book[:slots], book[slots : 2 * slots], book[2 * slots :]
+        call("tk_expert_sort", ids.data_ptr(), n * top, top, experts, max_tiles, slot_pair.data_ptr(), slot_token.data_ptr(),
+             tile_group.data_ptr(), _stream())
+        inter = torch.empty((slots, ff), dtype=h.dtype, device=h.device)
+        call("tk_grouped_gemm_bf16", h.data_ptr(), h.stride(0), slot_token.data_ptr(), None, tile_group.data_ptr(), max_tiles, 0,
+             0, 0, w_gate_up.data_ptr(), 2 * ff * width, inter.data_ptr(), ff, ff, width, slots, 1, 0, _stream())
+        y = torch.empty((n * top, width), dtype=h.dtype, device=h.device)
+        call("tk_grouped_gemm_bf16", inter.data_ptr(), ff, None, slot_pair.data_ptr(), tile_group.data_ptr(), max_tiles, 0,
+             0, 0, w_down.data_ptr(), width * ff, y.data_ptr(), width, width, ff, slots, 0, 0, _stream())
+        call("tk_expert_sum", h.data_ptr(), h.stride(0), y.data_ptr(), ids.data_ptr(), weights.data_ptr(),
+             shared.data_ptr() if shared is not None else None, shared_gate.data_ptr() if shared is not None else None,
+             out.data_ptr(), n, width, experts, top, _stream())
         return out
     inter = torch.empty((n * top, ff), dtype=h.dtype, device=h.device)
     call("tk_expert_gate_up", dtype_code(h.dtype), h.data_ptr(), h.stride(0), w_gate_up.data_ptr(), ids.data_ptr(),

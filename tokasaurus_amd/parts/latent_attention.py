@@ -61,7 +61,11 @@ class LatentAttention(Mixer):
         return CacheNeed(1, self.kv_rank, 0, 0)
 
     def check_cache(self, page_size: int, dtype: torch.dtype) -> None:
-        ops.check_attention_shape(dtype, self.num_heads, 1, self.kv_rank, page_size, value_dim=self.kv_rank, generic_only=True)
+        if ops.attention_tile_f32_fits(self.num_heads, 1, self.kv_rank, self.kv_rank, page_size):
+            ops.key_pages_shape(1, 1, page_size, self.kv_rank, padded=True)
+            ops.value_pages_shape(1, 1, page_size, self.kv_rank)
+        else:  # the plain kernel's bounds (heads times the latent's size)
+            ops.check_attention_shape(dtype, self.num_heads, 1, self.kv_rank, page_size, value_dim=self.kv_rank, generic_only=True)
 
     def load(self, tensors: dict[str, torch.Tensor], placer: Placer) -> None:
         for lin in (self.down, self.up_q, self.out):
