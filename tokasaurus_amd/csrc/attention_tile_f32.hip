@@ -34,13 +34,18 @@ struct __align__(sizeof(T) * 4) Raw4 { T v[4]; };
 // SPLIT: the NW wavefronts of a workgroup share one tile and take its key steps in turn
 // (wavefront w the steps w, w + NW, ..); they add up through LDS, always in wavefront order.
 // For steps of few tiles (single decoded tokens), whose walks would else be one long chain each.
-template <typename T, int KM, int VT, bool SPLIT, int NW>
+//
+// PART (with SPLIT): the keys are also cut into chunks of `chunk` keys at absolute multiples of it, a workgroup a
+// (tile, head block, chunk): blockIdx.z names the chunk.  A workgroup leaves its maxima, sums and weighted values
+// unnormalised in `part`; attention_tile_merge_kernel adds the chunks in ascending order.  For single decoded
+// tokens after long contexts, where a tile's walk would else keep one workgroup busy and the chip idle.
+template <typename T, int KM, int VT, bool SPLIT, int NW, bool PART = false>
 __global__ __launch_bounds__(NW * TK_WAVE) void attention_tile_f32_kernel(
     const T* __restrict__ q, int q_stride, T* __restrict__ out, int out_stride, const T* __restrict__ kcache,
     const T* __restrict__ vcache, const int* __restrict__ block_table, int table_stride,
     const int* __restrict__ q_start, const int* __restrict__ kv_len, const int* __restrict__ tile_req,
     const int* __restrict__ tile_row0, int nq, int nkv, int dk, int dv, int P, int window, float scale,
-    const float* __restrict__ sink, int gg) {
+    const float* __restrict__ sink, int gg, int chunk = 0, float* __restrict__ part = nullptr) {
   extern __shared__ float merge[];  // SPLIT: [waves][16] maxima, [waves][16] sums, [waves - 1][VT][4][64] weighted values
   const int lane = threadIdx.x & (TK_WAVE - 1), wave = threadIdx.x / TK_WAVE;
   const int group = nq / nkv;
@@ -63,8 +68,9 @@ __global__ __launch_bounds__(NW * TK_WAVE) void attention_tile_f32_kernel(
   const int n_tok = min(tt, q_end - row0);
   const int pos0 = kv - (q_end - row0);         // position of the tile's first token
   const int pos = pos0 + col / gg;              // of this column's token
-  const int last = pos0 + n_tok - 1;
-  const int lo_tile = window > 0 ? max(0, pos0 - window + 1) : 0;
+  const int last_all = pos0 + n_tok - 1;  // the last key any column of the tile sees
+  const int last = PART ? min(last_all, ((int)blockIdx.z + 1) * chunk - 1) : last_all;  // the last this workgroup walks
+  const int lo_tile = max(window > 0 ? max(0, pos0 - window + 1) : 0, PART ? (int)blockIdx.z * chunk : 0);
   const int* table = block_table + (size_t)r * table_stride;
   const int pieces = dk / 8;
   const size_t key_page = key_page_elems(P, dk);
@@ -157,7 +163,7 @@ __global__ __launch_bounds__(NW * TK_WAVE) void attention_tile_f32_kernel(
     float sc[4];
     float tmax = -INFINITY;
     // a step that every column of the tile sees whole needs no masks (the same for all lanes)
-    const bool whole = k0 + 15 <= pos0 && (window <= 0 || last - k0 < window) && n_tok * gg == 16;
+    const bool whole = k0 + 15 <= pos0 && (window <= 0 || last_all - k0 < window) && n_tok * gg == 16;
     if (whole) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
@@ -249,6 +255,20 @@ __global__ __launch_bounds__(NW * TK_WAVE) void attention_tile_f32_kernel(
     }
     m_run = m_all;
   }
+  if constexpr (PART) {
+    // [tile][head block][chunk]: 16 maxima, 16 sums, [VT][4][64] weighted values as the lanes hold them
+    const size_t unit = 32 + (size_t)VT * 4 * TK_WAVE;
+    float* dst = part + (((size_t)tile * gridDim.y + blockIdx.y) * gridDim.z + blockIdx.z) * unit;
+    if (c == 0) {
+      dst[col] = m_run;
+      dst[16 + col] = l;
+    }
+#pragma unroll
+    for (int t = 0; t < VT; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) dst[32 + (t * 4 + i) * TK_WAVE + lane] = o[t][i];
+    return;
+  }
   float keep = 1.f;
   if (sink && live) {
     // the sink joins the softmax like one more score: the maximum may rise to it
@@ -268,18 +288,85 @@ __global__ __launch_bounds__(NW * TK_WAVE) void attention_tile_f32_kernel(
   }
 }
 
+// One wavefront a (tile, head block): the chunks' partial results added in ascending order, then the sink and the
+// division, with the lanes' places as in the kernel above.
+template <typename T, int VT>
+__global__ __launch_bounds__(TK_WAVE) void attention_tile_merge_kernel(
+    const float* __restrict__ part, int chunks, T* __restrict__ out, int out_stride, const int* __restrict__ q_start,
+    const int* __restrict__ tile_req, const int* __restrict__ tile_row0, int nq, int nkv, int dv,
+    const float* __restrict__ sink, int gg) {
+  const int lane = threadIdx.x;
+  const int group = nq / nkv, blocks_per_kv = group / gg;
+  const int hb = blockIdx.y, tile = blockIdx.x;
+  const int head0 = (hb / blocks_per_kv) * group + (hb % blocks_per_kv) * gg;
+  const int col = lane & 15, c = lane >> 4;
+  const int tok = tile_row0[tile] + col / gg, head = head0 + col % gg;
+  const bool live = tok < q_start[tile_req[tile] + 1];
+  const size_t unit = 32 + (size_t)VT * 4 * TK_WAVE;
+  const float* src = part + ((size_t)tile * gridDim.y + hb) * chunks * unit;
+  float m_all = -INFINITY;
+  for (int z = 0; z < chunks; ++z) m_all = fmaxf(m_all, src[z * unit + col]);
+  float l = 0.f;
+  v4f o[VT];
+#pragma unroll
+  for (int t = 0; t < VT; ++t) o[t] = (v4f){0.f, 0.f, 0.f, 0.f};
+  for (int z = 0; z < chunks; ++z) {
+    const float mz = src[z * unit + col];
+    if (mz == -INFINITY) continue;  // a chunk none of whose keys this column sees
+    const float f = expf(mz - m_all);
+    l = fmaf(src[z * unit + 16 + col], f, l);
+#pragma unroll
+    for (int t = 0; t < VT; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[t][i] = fmaf(src[z * unit + 32 + (t * 4 + i) * TK_WAVE + lane], f, o[t][i]);
+  }
+  float keep = 1.f;
+  if (sink && live) {
+    const float sk = sink[head], m2 = fmaxf(m_all, sk);
+    keep = (m_all == -INFINITY) ? 0.f : expf(m_all - m2);
+    l = l * keep + expf(sk - m2);
+  }
+  if (!live) return;
+  const float inv = keep / l;
+  T* dst = out + (size_t)tok * out_stride + (size_t)head * dv;
+#pragma unroll
+  for (int t = 0; t < VT; ++t) {
+    if (16 * t < dv) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) dst[16 * t + 4 * c + i] = from_f32<T>(o[t][i] * inv);
+    }
+  }
+}
+
 // Whether this kernel takes the shape (else the caller uses the plain 32-bit kernel).
 TK_API int tk_attention_tile_f32_fits(int nq, int nkv, int dk, int dv, int P) {
   return (nq > 0 && nkv > 0 && nq % nkv == 0 && dk > 0 && dk % 8 == 0 && dk <= 32 * AT_MAX_KM && dv > 0 && dv % 16 == 0 &&
           dv <= 16 * AT_MAX_VT && P > 0 && P % 16 == 0) ? 1 : 0;
 }
 
+// 32-bit words of `part` that a (tile, head block, chunk) takes for a value head of dv elements
+TK_API int tk_attention_tile_part_words(int dv) {
+  const int vt = dv / 16;
+  const int VT = vt <= 2 ? 2 : (vt <= 4 ? 4 : (vt <= 8 ? 8 : 16));
+  return 32 + VT * 4 * TK_WAVE;
+}
+
 template <typename T, int KM, int VT>
 static void at_launch(dim3 grid, bool split, hipStream_t stream, const void* q, int q_stride, void* out, int out_stride,
                       const void* kcache, const void* vcache, const int* block_table, int table_stride,
                       const int* q_start, const int* kv_len, const int* tile_req, const int* tile_row0, int nq,
-                      int nkv, int dk, int dv, int P, int window, float scale, const float* sink, int gg) {
-  if (split) {
+                      int nkv, int dk, int dv, int P, int window, float scale, const float* sink, int gg, int chunk,
+                      float* part) {
+  if (split && chunk > 0) {
+    constexpr int NW = VT <= 4 ? 8 : 4;
+    const size_t smem = sizeof(float) * (NW * 32 + (size_t)(NW - 1) * VT * 4 * TK_WAVE);
+    hipLaunchKernelGGL((attention_tile_f32_kernel<T, KM, VT, true, NW, true>), grid, dim3(NW * TK_WAVE), smem, stream,
+                       (const T*)q, q_stride, (T*)out, out_stride, (const T*)kcache, (const T*)vcache, block_table,
+                       table_stride, q_start, kv_len, tile_req, tile_row0, nq, nkv, dk, dv, P, window, scale, sink, gg,
+                       chunk, part);
+    hipLaunchKernelGGL((attention_tile_merge_kernel<T, VT>), dim3(grid.x, grid.y), dim3(TK_WAVE), 0, stream, part, (int)grid.z,
+                       (T*)out, out_stride, q_start, tile_req, tile_row0, nq, nkv, dv, sink, gg);
+  } else if (split) {
     // eight wavefronts a tile where their sums fit the local memory, else four
     constexpr int NW = VT <= 4 ? 8 : 4;
     const size_t smem = sizeof(float) * (NW * 32 + (size_t)(NW - 1) * VT * 4 * TK_WAVE);
@@ -299,7 +386,7 @@ TK_API int tk_attention_tile_f32(int dt, const void* q, int q_stride, void* out,
                                  const void* vcache, const int* block_table, int table_stride, const int* q_start,
                                  const int* kv_len, const int* tile_req, const int* tile_row0, int n_tiles, int nq,
                                  int nkv, int dk, int dv, int P, int window, float scale, const float* sink, int gg,
-                                 int split, hipStream_t stream) {
+                                 int split, int chunk, int chunks, float* part, hipStream_t stream) {
   TK_REQUIRE(tk_attention_tile_f32_fits(nq, nkv, dk, dv, P), "attention_tile_f32: shape nq=%d nkv=%d dk=%d dv=%d P=%d not taken",
              nq, nkv, dk, dv, P);
   const int group = nq / nkv;
@@ -309,10 +396,13 @@ TK_API int tk_attention_tile_f32(int dt, const void* q, int q_stride, void* out,
   const int head_blocks = nkv * (group / gg);
   const int km = (dk + 31) / 32, vt = dv / 16;
   const bool sp = split != 0;
-  const dim3 grid(n_tiles, sp ? head_blocks : (head_blocks + AT_WAVES - 1) / AT_WAVES);
+  const bool parts = sp && chunk > 0;
+  TK_REQUIRE(!parts || (chunk % 128 == 0 && chunks > 0 && chunks < 65536 && part), "attention_tile_f32: chunks of a multiple of 128 keys, "
+             "their number and a place for their results");
+  const dim3 grid(n_tiles, sp ? head_blocks : (head_blocks + AT_WAVES - 1) / AT_WAVES, parts ? chunks : 1);
   TK_REQUIRE(grid.y < 65536, "attention_tile_f32: too many heads");
 #define AT_ARGS grid, sp, stream, q, q_stride, out, out_stride, kcache, vcache, block_table, table_stride, q_start, kv_len, \
-                tile_req, tile_row0, nq, nkv, dk, dv, P, window, scale, sink, gg
+                tile_req, tile_row0, nq, nkv, dk, dv, P, window, scale, sink, gg, parts ? chunk : 0, part
 #define AT_VT(T, KMV)                                      \
   do {                                                     \
     if (vt <= 2) at_launch<T, KMV, 2>(AT_ARGS);            \

@@ -1237,14 +1237,17 @@ def attention_tile_f32(
     q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, block_table: torch.Tensor, q_start: torch.Tensor,
     kv_len: torch.Tensor, tile_req: torch.Tensor, tile_row0: torch.Tensor, nq: int, nkv: int, key_dim: int,
     value_dim: int, page_size: int, heads_a_tile: int, window: int = 0, scale: float = 1.0,
-    sink: torch.Tensor | None = None, split: bool | None = None,
+    sink: torch.Tensor | None = None, split: bool | None = None, key_chunk: int = 0, longest: int = 0,
 ) -> torch.Tensor:
     """Attention in 32-bit arithmetic on the matrix cores: every token of the step over its
     request's pages; ``tile_req`` / ``tile_row0`` name each tile's request and its first token's
     row (a tile holds 16 / heads_a_tile neighbouring tokens of one request).  Window, scale,
     value size and sinks as in ``paged_attention_generic``; returns [tokens, nq * value_dim].
     ``split``: the four wavefronts of a workgroup share a tile and take its keys in turn (by
-    default when the step has so few tiles that their walks would leave the chip idle)."""
+    default when the step has so few tiles that their walks would leave the chip idle).
+    ``key_chunk`` (a multiple of 128; with ``longest``, a bound on every request's length that does not
+    depend on the batch): a split tile's keys are also cut at absolute multiples of ``key_chunk`` among
+    workgroups, whose partial results a second kernel adds in ascending order."""
     _gpu(q, kcache, vcache, block_table, q_start, kv_len, tile_req, tile_row0, sink)
     if split is None:
         split = tile_req.numel() * nkv * ((nq // nkv) // int(heads_a_tile)) < ATTENTION_TILE_SPLIT_BELOW
@@ -1258,11 +1261,16 @@ def attention_tile_f32(
           f"attention: the sinks must be contiguous float32 [{nq}]")
     _check_pages(kcache, vcache, nkv, page_size, key_dim, q.dtype, "attention", value_dim)
     out = torch.empty((q.shape[0], nq * value_dim), dtype=q.dtype, device=q.device)
+    chunks, part = 0, None
+    if split and key_chunk > 0 and longest > key_chunk:
+        chunks = -(-int(longest) // int(key_chunk))
+        words = load("core").tk_attention_tile_part_words(value_dim)
+        part = torch.empty((tile_req.numel() * nkv * ((nq // nkv) // int(heads_a_tile)) * chunks * words,), dtype=torch.float32, device=q.device)
     call("tk_attention_tile_f32", dtype_code(q.dtype), q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0),
          kcache.data_ptr(), vcache.data_ptr(), block_table.data_ptr(), block_table.stride(0), q_start.data_ptr(),
          kv_len.data_ptr(), tile_req.data_ptr(), tile_row0.data_ptr(), tile_req.numel(), nq, nkv, key_dim, value_dim,
          page_size, int(window), float(scale), sink.data_ptr() if sink is not None else None, int(heads_a_tile),
-         1 if split else 0, _stream())
+         1 if split else 0, int(key_chunk) if chunks else 0, chunks, part.data_ptr() if part is not None else None, _stream())
     return out
 
 

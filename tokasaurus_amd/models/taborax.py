@@ -37,7 +37,7 @@ def taborax_spec(cfg: TaboraxConfig) -> ModelSpec:
                 position = PartSpec("rotary_halves", {"dims": m.rot_dims, "base": m.rot_base})
             mixer = PartSpec("grouped_attention", {
                 "hidden_size": cfg.width, "num_heads": m.heads, "num_kv_heads": m.kv_heads, "key_dim": m.dim,
-                "value_dim": m.vdim, "scale": m.scale, "position": position, "sink_value": 0.0, "values_are_keys": True,
+                "value_dim": m.vdim, "scale": m.scale, "position": position, "sink_value": 0.0, "values_are_keys": True, "key_chunk": 256,
                 "names": {"q": f"{p}.q", "k": f"{p}.k", "o": f"{p}.o"}})
         params = {"mixer_norm": norm(f"l{i}.norm1"), "mixer": mixer, "mixer_post_norm": norm(f"l{i}.norm1b")}
         f, q = layer.ff, f"l{i}.mlp"

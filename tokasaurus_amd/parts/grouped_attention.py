@@ -75,6 +75,7 @@ class GroupedAttention(Mixer):
         shared: dict | None = None,
         sink_value: float | None = None,
         values_are_keys: bool = False,
+        key_chunk: int = 0,
     ):
         """``names``: checkpoint names of the q, k, v, o matrices (k and v only with ``own_kv``).
         ``projection_norm``: ``{"q": name, "k": name, "eps": eps}``, weights of the whole
@@ -83,7 +84,10 @@ class GroupedAttention(Mixer):
         keys (0: all): at least ``window``, more when another layer reads this cache further
         back; by default ``window``.  ``sink_name``: one number a query head.  ``sink_value``: no
         tensor, every head's sink has this score (0: one is added to the softmax's denominator).
-        ``values_are_keys``: ``names`` has no v; a token's values are its keys before the rotation."""
+        ``values_are_keys``: ``names`` has no v; a token's values are its keys before the rotation.
+        ``key_chunk``: in steps of few tokens a request's keys are cut at multiples of this many among
+        workgroups (0: never)."""
+        self.key_chunk = int(key_chunk)
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads are not a multiple of {num_kv_heads} kv heads")
         self.hidden_size, self.num_heads, self.num_kv_heads = hidden_size, num_heads, num_kv_heads
@@ -173,7 +177,8 @@ class GroupedAttention(Mixer):
             tile_req, tile_row0 = tile_plan(ctx, 16 // gg)
             attn = ops.attention_tile_f32(qkv, cache.keys, cache.values, cache.block_table, ctx.q_start, ctx.kv_len,
                                           tile_req, tile_row0, nq, nkv, dk, dv, cache.page_size, gg,
-                                          window=self.window, scale=self.scale, sink=self.sink)
+                                          window=self.window, scale=self.scale, sink=self.sink, key_chunk=self.key_chunk,
+                                          longest=ctx.extras.get("kv_bound", ctx.max_kv_len))
         else:  # sizes that the matrix-core kernel does not take
             attn = ops.paged_attention_generic(qkv, cache.keys, cache.values, cache.block_table, ctx.token_req, ctx.positions,
                                                nq, nkv, dk, cache.page_size, window=self.window, scale=self.scale,

@@ -33,10 +33,12 @@ from tokasaurus_amd.parts.linear import Linear, Placer
 @MIXERS.register("latent_attention")
 class LatentAttention(Mixer):
     def __init__(self, hidden_size: int, num_heads: int, key_dim: int, value_dim: int, q_rank: int, kv_rank: int, scale: float,
-                 norm_eps: float, names: dict[str, str]):
+                 norm_eps: float, names: dict[str, str], key_chunk: int = 256):
         """``names``: checkpoint names under the keys dq, dkv ([rank, hidden]), dq_norm, dkv_norm
         ([rank]), uq ([heads * key_dim, q_rank]), uk ([heads * key_dim, kv_rank]), uv
-        ([heads * value_dim, kv_rank]), o ([hidden, heads * value_dim])."""
+        ([heads * value_dim, kv_rank]), o ([hidden, heads * value_dim]).  ``key_chunk``: in steps of
+        few tokens a request's keys are cut at multiples of this many among workgroups (0: never)."""
+        self.key_chunk = int(key_chunk)
         self.hidden_size, self.num_heads = hidden_size, num_heads
         self.key_dim, self.value_dim, self.q_rank, self.kv_rank = int(key_dim), int(value_dim), int(q_rank), int(kv_rank)
         self.scale, self.norm_eps = float(scale), float(norm_eps)
@@ -97,7 +99,8 @@ class LatentAttention(Mixer):
             gg = ops.attention_tile_heads(H, ctx.max_q_len)
             tile_req, tile_row0 = tile_plan(ctx, 16 // gg)
             o = ops.attention_tile_f32(q, cache.keys, cache.values, cache.block_table, ctx.q_start, ctx.kv_len,
-                                       tile_req, tile_row0, H, 1, r, r, cache.page_size, gg, scale=self.scale)
+                                       tile_req, tile_row0, H, 1, r, r, cache.page_size, gg, scale=self.scale,
+                                       key_chunk=self.key_chunk, longest=ctx.extras.get("kv_bound", ctx.max_kv_len))
         else:
             o = ops.paged_attention_generic(q, cache.keys, cache.values, cache.block_table, ctx.token_req, ctx.positions,
                                             H, 1, r, cache.page_size, scale=self.scale, value_dim=r)
