@@ -127,7 +127,7 @@ TK_API int tk_qk_prepare(int dt, void* qkv, int row_stride, const int* positions
                          const float* k_weight, float eps, const float* freq, void* kcache, void* vcache,
                          int n_tokens, int nq, int nkv, int dq, int dk, int dv, int rot, int P, int write_cache,
                          int pair_half, int v_from_k, hipStream_t stream) {
-  TK_REQUIRE(n_tokens >= 0 && nq > 0 && nkv >= 0 && dq > 0 && dk > 0 && dv > 0 && P > 0,
+  TK_REQUIRE(n_tokens >= 0 && nq >= 0 && nkv >= 0 && nq + nkv > 0 && dq > 0 && dk > 0 && dv > 0 && P > 0,
              "qk_prepare: bad sizes tokens=%d nq=%d nkv=%d dq=%d dk=%d dv=%d P=%d", n_tokens, nq, nkv, dq, dk, dv, P);
   TK_REQUIRE(rot >= 0 && rot <= dk && rot <= dq && rot % 2 == 0, "qk_prepare: %d rotated elements of heads of %d and %d", rot, dq, dk);
   TK_REQUIRE(rot == 0 || freq, "qk_prepare: a rotation needs its frequencies");
@@ -146,5 +146,36 @@ TK_API int tk_qk_prepare(int dt, void* qkv, int row_stride, const int* positions
                        row_stride, positions, token_req, block_table, table_stride, q_weight, k_weight, eps,
                        freq, (bf16_t*)kcache, (bf16_t*)vcache, nq, nkv, dq, dk, dv, rot, P, write_cache, pair_half, v_from_k);
   TK_CHECK_LAUNCH("qk_prepare");
+  return 0;
+}
+
+// --------------------------------------------------------------------------
+// out[i, :] = the key of kv head `head` that request req[i] holds at position pos[i], read back from the pages:
+// for mixers that compute on cached keys outside the attention (a latent that is expanded for a prompt's portion).
+// --------------------------------------------------------------------------
+template <typename T>
+__global__ void gather_keys_kernel(const T* __restrict__ kcache, const int* __restrict__ block_table, int table_stride,
+                                   const int* __restrict__ req, const int* __restrict__ pos, T* __restrict__ out, int nkv,
+                                   int head, int dk, int P) {
+  const int i = blockIdx.x;
+  const int p = pos[i];
+  const int page = block_table[(size_t)req[i] * table_stride + p / P];
+  const T* src = kcache + ((size_t)page * nkv + head) * key_page_elems(P, dk);
+  for (int e = threadIdx.x; e < dk; e += blockDim.x) out[(size_t)i * dk + e] = src[key_offset(P, p % P, e)];
+}
+
+TK_API int tk_gather_keys(int dt, const void* kcache, const int* block_table, int table_stride, const int* req, const int* pos,
+                          void* out, int n, int nkv, int head, int dk, int P, hipStream_t stream) {
+  TK_REQUIRE(kcache && block_table && req && pos && out && n >= 0 && nkv > 0 && head >= 0 && head < nkv && dk > 0 && P > 0,
+             "gather_keys: bad arguments");
+  if (n == 0) return 0;
+  const int threads = dk >= 256 ? 256 : (dk >= 128 ? 128 : 64);
+  if (dt == TK_F32)
+    hipLaunchKernelGGL(gather_keys_kernel<float>, dim3(n), dim3(threads), 0, stream, (const float*)kcache, block_table, table_stride,
+                       req, pos, (float*)out, nkv, head, dk, P);
+  else
+    hipLaunchKernelGGL(gather_keys_kernel<bf16_t>, dim3(n), dim3(threads), 0, stream, (const bf16_t*)kcache, block_table,
+                       table_stride, req, pos, (bf16_t*)out, nkv, head, dk, P);
+  TK_CHECK_LAUNCH("gather_keys");
   return 0;
 }

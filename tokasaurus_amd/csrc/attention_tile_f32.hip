@@ -288,14 +288,15 @@ __global__ __launch_bounds__(NW * TK_WAVE) void attention_tile_f32_kernel(
   }
 }
 
-// One wavefront a (tile, head block): the chunks' partial results added in ascending order, then the sink and the
-// division, with the lanes' places as in the kernel above.
+// A workgroup a (tile, head block), a wavefront a block of 16 value elements: the chunks' partial results added in
+// ascending order, then the sink and the division, with the lanes' places as in the kernel above.
 template <typename T, int VT>
-__global__ __launch_bounds__(TK_WAVE) void attention_tile_merge_kernel(
+__global__ __launch_bounds__(VT * TK_WAVE) void attention_tile_merge_kernel(
     const float* __restrict__ part, int chunks, T* __restrict__ out, int out_stride, const int* __restrict__ q_start,
     const int* __restrict__ tile_req, const int* __restrict__ tile_row0, int nq, int nkv, int dv,
     const float* __restrict__ sink, int gg) {
-  const int lane = threadIdx.x;
+  const int lane = threadIdx.x & (TK_WAVE - 1), t = threadIdx.x / TK_WAVE;
+  if (16 * t >= dv) return;
   const int group = nq / nkv, blocks_per_kv = group / gg;
   const int hb = blockIdx.y, tile = blockIdx.x;
   const int head0 = (hb / blocks_per_kv) * group + (hb % blocks_per_kv) * gg;
@@ -305,20 +306,22 @@ __global__ __launch_bounds__(TK_WAVE) void attention_tile_merge_kernel(
   const size_t unit = 32 + (size_t)VT * 4 * TK_WAVE;
   const float* src = part + ((size_t)tile * gridDim.y + hb) * chunks * unit;
   float m_all = -INFINITY;
+#pragma unroll 8
   for (int z = 0; z < chunks; ++z) m_all = fmaxf(m_all, src[z * unit + col]);
   float l = 0.f;
-  v4f o[VT];
-#pragma unroll
-  for (int t = 0; t < VT; ++t) o[t] = (v4f){0.f, 0.f, 0.f, 0.f};
+  v4f o = (v4f){0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
   for (int z = 0; z < chunks; ++z) {
     const float mz = src[z * unit + col];
-    if (mz == -INFINITY) continue;  // a chunk none of whose keys this column sees
-    const float f = expf(mz - m_all);
-    l = fmaf(src[z * unit + 16 + col], f, l);
+    const float lz = src[z * unit + 16 + col];
+    v4f oz;
 #pragma unroll
-    for (int t = 0; t < VT; ++t)
+    for (int i = 0; i < 4; ++i) oz[i] = src[z * unit + 32 + (t * 4 + i) * TK_WAVE + lane];
+    // a chunk none of whose keys this column sees (maximum -inf, sums zero) adds nothing
+    const float f = (mz == -INFINITY) ? 0.f : expf(mz - m_all);
+    l = fmaf(lz, f, l);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) o[t][i] = fmaf(src[z * unit + 32 + (t * 4 + i) * TK_WAVE + lane], f, o[t][i]);
+    for (int i = 0; i < 4; ++i) o[i] = fmaf(oz[i], f, o[i]);
   }
   float keep = 1.f;
   if (sink && live) {
@@ -330,12 +333,7 @@ __global__ __launch_bounds__(TK_WAVE) void attention_tile_merge_kernel(
   const float inv = keep / l;
   T* dst = out + (size_t)tok * out_stride + (size_t)head * dv;
 #pragma unroll
-  for (int t = 0; t < VT; ++t) {
-    if (16 * t < dv) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) dst[16 * t + 4 * c + i] = from_f32<T>(o[t][i] * inv);
-    }
-  }
+  for (int i = 0; i < 4; ++i) dst[16 * t + 4 * c + i] = from_f32<T>(o[i] * inv);
 }
 
 // Whether this kernel takes the shape (else the caller uses the plain 32-bit kernel).
@@ -364,7 +362,7 @@ static void at_launch(dim3 grid, bool split, hipStream_t stream, const void* q, 
                        (const T*)q, q_stride, (T*)out, out_stride, (const T*)kcache, (const T*)vcache, block_table,
                        table_stride, q_start, kv_len, tile_req, tile_row0, nq, nkv, dk, dv, P, window, scale, sink, gg,
                        chunk, part);
-    hipLaunchKernelGGL((attention_tile_merge_kernel<T, VT>), dim3(grid.x, grid.y), dim3(TK_WAVE), 0, stream, part, (int)grid.z,
+    hipLaunchKernelGGL((attention_tile_merge_kernel<T, VT>), dim3(grid.x, grid.y), dim3(VT * TK_WAVE), 0, stream, part, (int)grid.z,
                        (T*)out, out_stride, q_start, tile_req, tile_row0, nq, nkv, dv, sink, gg);
   } else if (split) {
     // eight wavefronts a tile where their sums fit the local memory, else four

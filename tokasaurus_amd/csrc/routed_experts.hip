@@ -38,13 +38,42 @@ __device__ __forceinline__ float wave_dot(const T* __restrict__ w, const T* __re
   return wave_sum(acc);
 }
 
+// The same for two rows of weights against one x, in one pass (each sum in the order wave_dot has).
+template <typename T>
+__device__ __forceinline__ void wave_dot2(const T* __restrict__ w0, const T* __restrict__ w1, const T* __restrict__ x, int n,
+                                          float& d0, float& d1) {
+  constexpr int V = 16 / sizeof(T);
+  const int lane = threadIdx.x & (TK_WAVE - 1);
+  float a0 = 0.f, a1 = 0.f;
+  if (n % V == 0 && (((uintptr_t)w0 | (uintptr_t)w1 | (uintptr_t)x) & 15) == 0) {
+    for (int i = lane * V; i < n; i += TK_WAVE * V) {
+      const uint4 wa = *(const uint4*)(w0 + i), wb = *(const uint4*)(w1 + i), xa = *(const uint4*)(x + i);
+      const T* wp = (const T*)&wa;
+      const T* wq = (const T*)&wb;
+      const T* xp = (const T*)&xa;
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        a0 = fmaf(to_f32<T>(wp[e]), to_f32<T>(xp[e]), a0);
+        a1 = fmaf(to_f32<T>(wq[e]), to_f32<T>(xp[e]), a1);
+      }
+    }
+  } else {
+    for (int i = lane; i < n; i += TK_WAVE) {
+      a0 = fmaf(to_f32<T>(w0[i]), to_f32<T>(x[i]), a0);
+      a1 = fmaf(to_f32<T>(w1[i]), to_f32<T>(x[i]), a1);
+    }
+  }
+  d0 = wave_sum(a0);
+  d1 = wave_sum(a1);
+}
+
 // --------------------------------------------------------------------------
 // The router.  One workgroup a token.  n_all = routed + identity experts.  ids [tokens, top] names
 // the chosen experts in the order of their choice scores, weights [tokens, top] their softmax
 // scores (the correction moves the choice, not the weight).
 // --------------------------------------------------------------------------
 template <typename T>
-__global__ __launch_bounds__(256) void expert_route_kernel(
+__global__ __launch_bounds__(1024) void expert_route_kernel(
     const T* __restrict__ h, int h_stride, const T* __restrict__ w_router, const float* __restrict__ correction,
     const T* __restrict__ w_gate, int width, int n_all, int groups, int keep, int top, int* __restrict__ ids,
     float* __restrict__ weights, float* __restrict__ shared_gate) {
@@ -137,12 +166,14 @@ TK_API int tk_expert_route(int dt, const void* h, int h_stride, const void* w_ro
   const size_t smem = sizeof(float) * (size_t)(2 * n_all + groups);
   TK_REQUIRE(smem <= 48 * 1024, "expert_route: %d experts do not fit the local memory", n_all);
   if (tokens == 0) return 0;
+  // a wavefront a logit where the step has few tokens (each dot product is a chain of loads), four wavefronts for many
+  const int threads = tokens <= 64 ? 1024 : 256;
   if (dt == TK_F32)
-    hipLaunchKernelGGL(expert_route_kernel<float>, dim3(tokens), dim3(256), smem, stream, (const float*)h, h_stride,
+    hipLaunchKernelGGL(expert_route_kernel<float>, dim3(tokens), dim3(threads), smem, stream, (const float*)h, h_stride,
                        (const float*)w_router, correction, (const float*)w_gate, width, n_all, groups, keep, top, ids,
                        weights, shared_gate);
   else
-    hipLaunchKernelGGL(expert_route_kernel<bf16_t>, dim3(tokens), dim3(256), smem, stream, (const bf16_t*)h, h_stride,
+    hipLaunchKernelGGL(expert_route_kernel<bf16_t>, dim3(tokens), dim3(threads), smem, stream, (const bf16_t*)h, h_stride,
                        (const bf16_t*)w_router, correction, (const bf16_t*)w_gate, width, n_all, groups, keep, top, ids,
                        weights, shared_gate);
   TK_CHECK_LAUNCH("expert_route");
@@ -154,7 +185,7 @@ TK_API int tk_expert_route(int dt, const void* h, int h_stride, const void* w_ro
 // expert (others are skipped).  w_gate_up: [experts][2 * ff][width], gate rows first.
 // Workgroup (pair, block of EX_ROWS outputs), a wavefront an output at a time.
 // --------------------------------------------------------------------------
-#define EX_ROWS 16
+#define EX_ROWS 4  // one output a wavefront: a step of few tokens is a chain of loads, so many short workgroups
 template <typename T>
 __global__ __launch_bounds__(256) void expert_gate_up_kernel(
     const T* __restrict__ h, int h_stride, const T* __restrict__ w_gate_up, const int* __restrict__ ids,
@@ -168,8 +199,8 @@ __global__ __launch_bounds__(256) void expert_gate_up_kernel(
   const T* wu = wg + (size_t)ff * width;
   const int j0 = blockIdx.y * EX_ROWS;
   for (int j = j0 + wave; j < min(j0 + EX_ROWS, ff); j += nwaves) {
-    const float g = wave_dot<T>(wg + (size_t)j * width, row, width);
-    const float u = wave_dot<T>(wu + (size_t)j * width, row, width);
+    float g, u;
+    wave_dot2<T>(wg + (size_t)j * width, wu + (size_t)j * width, row, width, g, u);
     if (lane == 0) {
       // gate, up and the activation as the storage type sees them, as the dense feed-forward's epilogue
       const float gr = round_to<T>(g), ur = round_to<T>(u);

@@ -42,6 +42,7 @@ _SIGNATURES: dict[str, dict[str, list]] = {
         "tk_residual_norm": [c_int, _P, _P, _P, c_float, _P, _P, _P, c_float, c_float, _P, _P, c_int, c_int, _P],
         "tk_softcap": [_P, c_size_t, c_float, _P],
         "tk_qk_prepare": [c_int, _P, c_int, _P, _P, _P, c_int, _P, _P, c_float, _P, _P, _P] + [c_int] * 11 + [_P],
+        "tk_gather_keys": [c_int, _P, _P, c_int, _P, _P, _P] + [c_int] * 5 + [_P],
         "tk_post_norm_residual": [c_int, _P, _P, _P, c_float, _P, _P, c_float, _P, c_int, c_int, _P],
         "tk_concat_cast": [c_int, _P, _P, _P, c_int, c_int, _P],
         "tk_expert_route": [c_int, _P, c_int, _P, _P, _P] + [c_int] * 6 + [_P, _P, _P, _P],

@@ -1212,6 +1212,23 @@ def qk_prepare(
          1 if pair_halves else 0, 1 if values_are_keys else 0, _stream())
 
 
+def gather_keys(kcache: torch.Tensor, block_table: torch.Tensor, req: torch.Tensor, pos: torch.Tensor, key_dim: int,
+                page_size: int, head: int = 0) -> torch.Tensor:
+    """The keys of kv head ``head`` that request ``req[i]`` (a row of ``block_table``) holds at position
+    ``pos[i]``, read back from the pages: [len(req), key_dim]."""
+    _gpu(kcache, block_table, req, pos)
+    for t, name in ((block_table, "block_table"), (req, "req"), (pos, "pos")):
+        _i32(t, name)
+    nkv = kcache.shape[1]
+    _need(kcache.is_contiguous() and kcache.shape[1:] == key_pages_shape(1, nkv, page_size, key_dim, padded=True)[1:],
+          "gather_keys: key pages of this head size and page size")
+    _need(block_table.dim() == 2 and req.numel() == pos.numel(), "gather_keys: block_table [requests, width], one request and one position a row")
+    out = torch.empty((req.numel(), key_dim), dtype=kcache.dtype, device=kcache.device)
+    call("tk_gather_keys", dtype_code(kcache.dtype), kcache.data_ptr(), block_table.data_ptr(), block_table.stride(0), req.data_ptr(),
+         pos.data_ptr(), out.data_ptr(), req.numel(), nkv, int(head), key_dim, page_size, _stream())
+    return out
+
+
 def attention_tile_f32_fits(nq: int, nkv: int, key_dim: int, value_dim: int, page_size: int) -> bool:
     """Whether the 32-bit matrix-core attention takes the shape (key size a multiple of 8 up to
     256, value size a multiple of 16 up to 256, pages of a multiple of 16 keys)."""
@@ -1237,7 +1254,7 @@ def attention_tile_f32(
     q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, block_table: torch.Tensor, q_start: torch.Tensor,
     kv_len: torch.Tensor, tile_req: torch.Tensor, tile_row0: torch.Tensor, nq: int, nkv: int, key_dim: int,
     value_dim: int, page_size: int, heads_a_tile: int, window: int = 0, scale: float = 1.0,
-    sink: torch.Tensor | None = None, split: bool | None = None, key_chunk: int = 0, longest: int = 0,
+    sink: torch.Tensor | None = None, split: bool | None = None, key_chunk: int = 0, longest: int = 0, first_row: int = 0,
 ) -> torch.Tensor:
     """Attention in 32-bit arithmetic on the matrix cores: every token of the step over its
     request's pages; ``tile_req`` / ``tile_row0`` name each tile's request and its first token's
@@ -1247,7 +1264,9 @@ def attention_tile_f32(
     default when the step has so few tiles that their walks would leave the chip idle).
     ``key_chunk`` (a multiple of 128; with ``longest``, a bound on every request's length that does not
     depend on the batch): a split tile's keys are also cut at absolute multiples of ``key_chunk`` among
-    workgroups, whose partial results a second kernel adds in ascending order."""
+    workgroups, whose partial results a second kernel adds in ascending order.
+    ``first_row``: ``q`` holds the step's rows from this one on only (the tiles name none before it), and so
+    does the result."""
     _gpu(q, kcache, vcache, block_table, q_start, kv_len, tile_req, tile_row0, sink)
     if split is None:
         split = tile_req.numel() * nkv * ((nq // nkv) // int(heads_a_tile)) < ATTENTION_TILE_SPLIT_BELOW
@@ -1266,7 +1285,10 @@ def attention_tile_f32(
         chunks = -(-int(longest) // int(key_chunk))
         words = load("core").tk_attention_tile_part_words(value_dim)
         part = torch.empty((tile_req.numel() * nkv * ((nq // nkv) // int(heads_a_tile)) * chunks * words,), dtype=torch.float32, device=q.device)
-    call("tk_attention_tile_f32", dtype_code(q.dtype), q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0),
+    # the kernel finds a tile's rows by their place in the step
+    q_base = q.data_ptr() - int(first_row) * q.stride(0) * q.element_size()
+    out_base = out.data_ptr() - int(first_row) * out.stride(0) * out.element_size()
+    call("tk_attention_tile_f32", dtype_code(q.dtype), q_base, q.stride(0), out_base, out.stride(0),
          kcache.data_ptr(), vcache.data_ptr(), block_table.data_ptr(), block_table.stride(0), q_start.data_ptr(),
          kv_len.data_ptr(), tile_req.data_ptr(), tile_row0.data_ptr(), tile_req.numel(), nq, nkv, key_dim, value_dim,
          page_size, int(window), float(scale), sink.data_ptr() if sink is not None else None, int(heads_a_tile),

@@ -6,14 +6,23 @@ Per token: the query latent ``cq = norm(W_dq h)`` and the key/value latent ``c =
 ``score = (q . k) * scale`` over every earlier token and the token itself, an ordinary softmax,
 no positions; the output projection reads the heads side by side.
 
-The engine never expands a cached token's keys or values.  Since ``q_h . (W_uk,h c) =
-(W_uk,h^T q_h) . c`` and ``sum_j p_j W_uv,h c_j = W_uv,h sum_j p_j c_j``, a head's query is taken
-into the latent's space (a matrix a head, ``ops.head_linear``), the attention runs with ONE
-key/value head whose keys and values are both the latent (every query head reads it: the
-arithmetic intensity of the cache is that of ``num_heads`` queries a key), and the head's
-result is taken from the latent's space to its values by ``W_uv,h``.  The pages hold the
-latent twice, once in the key layout and once in the value layout, ``2 * kv_rank`` numbers a
-token and layer where expanded keys and values would take ``num_heads * (key_dim + value_dim)``.
+Two forms of the same sums, chosen request by request in every step:
+
+* **Single tokens** never expand a cached token's keys or values.  Since ``q_h . (W_uk,h c) =
+  (W_uk,h^T q_h) . c`` and ``sum_j p_j W_uv,h c_j = W_uv,h sum_j p_j c_j``, a head's query is taken
+  into the latent's space (a matrix a head, ``ops.head_linear``), the attention runs with ONE
+  key/value head whose keys and values are both the latent (every query head reads it: the
+  arithmetic intensity of the cache is that of ``num_heads`` queries a key), and the head's
+  result is taken from the latent's space to its values by ``W_uv,h``.
+* **Portions of prompts** expand: in the latent's space a score costs ``kv_rank`` multiply-adds
+  a head instead of ``key_dim``, which for many queries outweighs expanding every key once.  The
+  latents of the portion's requests are read back from the pages (``ops.gather_keys``), one
+  product gives all heads' keys and values, and they go into pages of the step's own (a block
+  table that counts up) over which the ordinary attention runs.  Nothing of it is kept.
+
+The pages hold the latent twice, once in the key layout and once in the value layout,
+``2 * kv_rank`` numbers a token and layer where expanded keys and values would take
+``num_heads * (key_dim + value_dim)``.
 
 Scores, softmax weights and norms are 32-bit arithmetic in either storage type; the kernels are
 those of ``grouped_attention`` (``ops.qk_prepare`` norms both latents and appends,
@@ -22,9 +31,11 @@ those of ``grouped_attention`` (``ops.qk_prepare`` norms both latents and append
 
 from __future__ import annotations
 
+import numpy as np
 import torch
 
 from tokasaurus_amd.kernels import ops
+from tokasaurus_amd.kernels.upload import upload
 from tokasaurus_amd.parts.base import MATRIX, MIXERS, NORM_WEIGHT, CacheNeed, CacheView, Mixer, StepContext, TensorSpec
 from tokasaurus_amd.parts.grouped_attention import tile_plan
 from tokasaurus_amd.parts.linear import Linear, Placer
@@ -46,17 +57,17 @@ class LatentAttention(Mixer):
         self.down = Linear(hidden_size, [names["dq"], names["dkv"]], [self.q_rank, self.kv_rank])
         self.up_q = Linear(self.q_rank, [names["uq"]], [num_heads * self.key_dim])
         self.out = Linear(num_heads * self.value_dim, [names["o"]], [hidden_size])
+        # all heads' keys and values of a latent in one product (prompt portions)
+        self.expand = Linear(self.kv_rank, [names["uk"], names["uv"]], [num_heads * self.key_dim, num_heads * self.value_dim])
         self.q_norm_weight = self.c_norm_weight = None
         self.to_latent: torch.Tensor | None = None  # [heads, kv_rank, key_dim]: W_uk,h transposed
         self.from_latent: torch.Tensor | None = None  # [heads, value_dim, kv_rank]: W_uv,h
 
     def tensor_specs(self) -> list[TensorSpec]:
         n, H = self.names, self.num_heads
-        return self.down.tensor_specs() + self.up_q.tensor_specs() + self.out.tensor_specs() + [
+        return self.down.tensor_specs() + self.up_q.tensor_specs() + self.out.tensor_specs() + self.expand.tensor_specs() + [
             TensorSpec(n["dq_norm"], (self.q_rank,), NORM_WEIGHT),
             TensorSpec(n["dkv_norm"], (self.kv_rank,), NORM_WEIGHT),
-            TensorSpec(n["uk"], (H * self.key_dim, self.kv_rank), MATRIX),
-            TensorSpec(n["uv"], (H * self.value_dim, self.kv_rank), MATRIX),
         ]
 
     def cache_need(self) -> CacheNeed:
@@ -70,7 +81,7 @@ class LatentAttention(Mixer):
             ops.check_attention_shape(dtype, self.num_heads, 1, self.kv_rank, page_size, value_dim=self.kv_rank, generic_only=True)
 
     def load(self, tensors: dict[str, torch.Tensor], placer: Placer) -> None:
-        for lin in (self.down, self.up_q, self.out):
+        for lin in (self.down, self.up_q, self.out, self.expand):
             lin.load(tensors, placer)
         n, H = self.names, self.num_heads
 
@@ -94,19 +105,67 @@ class LatentAttention(Mixer):
         cq = lat[:, : self.q_rank]
         if lat.dtype != torch.float32 and (self.q_rank % 8 or lat.stride(0) % 8):
             cq = torch.empty((lat.shape[0], self.q_rank), dtype=lat.dtype, device=lat.device).copy_(cq)
-        q = ops.head_linear(self.up_q(cq), self.to_latent)  # [tokens, heads * kv_rank]
-        if ops.attention_tile_f32_fits(H, 1, r, r, cache.page_size):
-            gg = ops.attention_tile_heads(H, ctx.max_q_len)
-            tile_req, tile_row0 = tile_plan(ctx, 16 // gg)
-            o = ops.attention_tile_f32(q, cache.keys, cache.values, cache.block_table, ctx.q_start, ctx.kv_len,
-                                       tile_req, tile_row0, H, 1, r, r, cache.page_size, gg, scale=self.scale,
-                                       key_chunk=self.key_chunk, longest=ctx.extras.get("kv_bound", ctx.max_kv_len))
+        q = self.up_q(cq)  # [tokens, heads * key_dim]
+        # the requests that bring portions come first in a step; their tokens are the step's first rows
+        portions = int(ctx.extras.get("num_portions", 0))
+        first_single = ctx.host_q_start[portions] if portions else 0
+        if portions and ops.attention_tile_f32_fits(H, H, self.key_dim, self.value_dim, cache.page_size):
+            o = self._over_expanded(q, ctx, cache, portions)
+            if first_single < ctx.num_tokens:
+                o[first_single:] = self._over_latent(q[first_single:], ctx, cache, first_single, ctx.num_requests - portions)
         else:
-            o = ops.paged_attention_generic(q, cache.keys, cache.values, cache.block_table, ctx.token_req, ctx.positions,
-                                            H, 1, r, cache.page_size, scale=self.scale, value_dim=r)
-        if rows is not None:
-            o = ops.gather_rows(o, rows)
-        return ops.head_linear(o, self.from_latent)  # [tokens, heads * value_dim]
+            o = self._over_latent(q, ctx, cache, 0, None)
+        return o if rows is None else ops.gather_rows(o, rows)
+
+    def _over_latent(self, q: torch.Tensor, ctx: StepContext, cache: CacheView, first_row: int, last_requests: int | None) -> torch.Tensor:
+        """Attention in the latent's space for the step's rows from ``first_row`` on (``q`` holds those
+        rows), which belong to the step's last ``last_requests`` requests, one token each (None: all
+        rows of all requests)."""
+        H, r = self.num_heads, self.kv_rank
+        ql = ops.head_linear(q, self.to_latent)  # [rows, heads * kv_rank]
+        if ops.attention_tile_f32_fits(H, 1, r, r, cache.page_size):
+            gg = ops.attention_tile_heads(H, ctx.max_q_len if last_requests is None else 1)
+            tile_req, tile_row0 = tile_plan(ctx, 16 // gg)
+            if last_requests is not None:  # a request of one token is one tile, whatever a tile holds
+                tile_req, tile_row0 = tile_req[tile_req.numel() - last_requests:], tile_row0[tile_row0.numel() - last_requests:]
+            o = ops.attention_tile_f32(ql, cache.keys, cache.values, cache.block_table, ctx.q_start, ctx.kv_len,
+                                       tile_req, tile_row0, H, 1, r, r, cache.page_size, gg, scale=self.scale,
+                                       key_chunk=self.key_chunk, longest=ctx.extras.get("kv_bound", ctx.max_kv_len),
+                                       first_row=first_row)
+        else:
+            o = ops.paged_attention_generic(ql, cache.keys, cache.values, cache.block_table, ctx.token_req[first_row:],
+                                            ctx.positions[first_row:], H, 1, r, cache.page_size, scale=self.scale, value_dim=r)
+        return ops.head_linear(o, self.from_latent)  # [rows, heads * value_dim]
+
+    def _over_expanded(self, q: torch.Tensor, ctx: StepContext, cache: CacheView, portions: int) -> torch.Tensor:
+        """Attention over expanded keys and values for the tokens of the step's first ``portions``
+        requests; returns rows for all of the step's tokens, of which only those are written."""
+        H, dk, dv, P = self.num_heads, self.key_dim, self.value_dim, cache.page_size
+        plan = ctx.extras.get(("expanded_keys_plan", portions, P))
+        if plan is None:  # made once a step, shared by the layers
+            lens = np.asarray(ctx.host_kv_len[:portions], dtype=np.int64)
+            pages = -(-lens // P)
+            first_page = np.concatenate([[0], np.cumsum(pages)])
+            total = int(lens.sum())
+            req = np.repeat(np.arange(portions, dtype=np.int32), lens)
+            pos = (np.arange(total, dtype=np.int64) - np.repeat(np.concatenate([[0], np.cumsum(lens)[:-1]]), lens)).astype(np.int32)
+            table = np.zeros((portions, int(pages.max())), dtype=np.int32)
+            for i in range(portions):
+                table[i, : pages[i]] = first_page[i] + np.arange(pages[i])
+            dev = upload(np.concatenate([req, pos, table.reshape(-1)]), torch.int32, q.device)
+            n_tiles = sum(-(-(ctx.host_q_start[i + 1] - ctx.host_q_start[i]) // 16) for i in range(portions))
+            plan = ctx.extras[("expanded_keys_plan", portions, P)] = (
+                dev[:total], dev[total : 2 * total], dev[2 * total :].view(portions, -1), int(first_page[-1]), n_tiles)
+        req_d, pos_d, table_d, n_pages, n_tiles = plan
+        latents = ops.gather_keys(cache.keys, cache.block_table, req_d, pos_d, self.kv_rank, P)
+        kv = self.expand(latents)  # [all keys of these requests, heads * key_dim | heads * value_dim]
+        # (zeros: the rest of a request's last page is read, with weight zero, and must hold numbers)
+        keys = torch.zeros(ops.key_pages_shape(n_pages, H, P, dk, padded=True), dtype=q.dtype, device=q.device)
+        values = torch.zeros(ops.value_pages_shape(n_pages, H, P, dv), dtype=q.dtype, device=q.device)
+        ops.qk_prepare(kv, pos_d, req_d, table_d, None, None, 0.0, None, keys, values, 0, H, dk, dv, P)
+        tile_req, tile_row0 = tile_plan(ctx, 16)
+        return ops.attention_tile_f32(q, keys, values, table_d, ctx.q_start, ctx.kv_len, tile_req[:n_tiles], tile_row0[:n_tiles],
+                                      H, H, dk, dv, P, 1, scale=self.scale)
 
     def mix(self, h, ctx, cache, state, rows, out_f32: bool = False):
         return self.out(self._attend(h, ctx, cache, rows), out_f32=out_f32)
