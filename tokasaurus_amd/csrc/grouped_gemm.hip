@@ -8,7 +8,7 @@
 //                         silu(gate) * up of two halves of W[g]
 //   tk_expert_sum         per token the weighted sum of its pairs' rows, identity experts, shared expert
 //
-// A wavefront owns GG_TM = 32 slots x 64 outputs (32 in the gated form, for each of gate and up): weight rows
+// A wavefront owns GG_TM = 64 slots x 64 outputs (32 in the gated form, for each of gate and up): weight rows
 // are the first operand of the matrix core, read straight from memory 16 bytes a lane, the slots' rows the
 // second; a lane ends up with 4 neighbouring outputs of one slot.  The next step's operands are asked for
 // before the current step's products.  Sums are 32-bit and run over k in ascending order for every output:
@@ -20,7 +20,7 @@
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
-#define GG_TM 32
+#define GG_TM 64
 #define GG_WAVES 4
 
 __device__ __forceinline__ bf16x8_t gg_zero8() {

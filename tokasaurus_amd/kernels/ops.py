@@ -1236,6 +1236,8 @@ def attention_tile_f32_fits(nq: int, nkv: int, key_dim: int, value_dim: int, pag
 
 
 ATTENTION_TILE_SPLIT_BELOW = 2048  # (tile, head block) pairs of a step below which the wavefronts share tiles
+ATTENTION_TILE_WORKGROUPS = 512  # workgroups a step with key chunks should have before its chunks grow
+ATTENTION_TILE_LONGEST_CHUNK = 2048
 
 
 def attention_tile_heads(group: int, max_q_len: int) -> int:
@@ -1282,6 +1284,11 @@ def attention_tile_f32(
     out = torch.empty((q.shape[0], nq * value_dim), dtype=q.dtype, device=q.device)
     chunks, part = 0, None
     if split and key_chunk > 0 and longest > key_chunk:
+        # longer chunks where the step has workgroups enough without short ones: a chunk's walk should be long
+        # enough to hide its first loads
+        groups = tile_req.numel() * nkv * ((nq // nkv) // int(heads_a_tile))
+        while key_chunk < ATTENTION_TILE_LONGEST_CHUNK and groups * -(-int(longest) // (2 * key_chunk)) >= ATTENTION_TILE_WORKGROUPS:
+            key_chunk *= 2
         chunks = -(-int(longest) // int(key_chunk))
         words = load("core").tk_attention_tile_part_words(value_dim)
         part = torch.empty((tile_req.numel() * nkv * ((nq // nkv) // int(heads_a_tile)) * chunks * words,), dtype=torch.float32, device=q.device)
@@ -1456,7 +1463,7 @@ def squared_relu_(x: torch.Tensor) -> torch.Tensor:
 # a matrix a head; experts of which a token uses a few
 # --------------------------------------------------------------------------
 
-GROUPED_TILE = 32  # slots a tile of the grouped matrix-core product (GG_TM of grouped_gemm.hip)
+GROUPED_TILE = 64  # slots a tile of the grouped matrix-core product (GG_TM of grouped_gemm.hip)
 GROUPED_FROM_ROWS = 16  # rows above which the products of experts and of heads run in tiles on the matrix cores
 
 
