@@ -68,10 +68,10 @@ STRAIGHT = {
         attention_layer(3, 3, 40, 0.15, rot={"base": 10000.0, "dims": 6}, mlp=dense(120)),
     ],
 }
-# sizes that fit nothing: a width, ranks, expert and feed-forward sizes and a vocabulary that are no multiples of 8
+# sizes that fit nothing: a width (no multiple of 4), ranks, expert and feed-forward sizes and a vocabulary that are no multiples of 8
 # (or of 2); the loop starts at the first layer; one group of two kept; a single head over an odd latent
 AWKWARD = {
-    "architecture": "Taborax", "vocab": 131, "width": 100, "norm": {"eps": 1e-4},
+    "architecture": "Taborax", "vocab": 131, "width": 90, "norm": {"eps": 1e-4},
     "loop": {"start": 0, "stop": 2, "times": 2},
     "layers": [
         latent_layer(3, 12, 20, 10, 36, 0.3, moe(20, 9, 2, identity=3, groups=(2, 1), shared=30)),

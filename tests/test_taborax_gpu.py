@@ -140,6 +140,7 @@ SINGLE_LAYERS = {
     "latent_one_head_odd_sizes": latent_layer(1, 12, 7, 9, 21, 0.3),
     "latent_sizes_of_a_large_model": latent_layer(4, 64, 64, 72, 128, 0.12, dense(96)),
     "latent_beyond_the_matrix_core_kernel": latent_layer(2, 16, 16, 24, 272, 0.1),
+    "latent_more_heads_than_the_plain_kernel_takes_at_once": latent_layer(9, 8, 16, 16, 264, 0.1),
     "attention_halves_of_a_part": attention_layer(4, 2, 32, 0.18, rot={"base": 100.0, "dims": 12}),
     "attention_whole_head_no_grouping": attention_layer(3, 3, 8, 0.4, rot={"base": 9.0, "dims": 8}),
     "attention_no_rotation_odd_head": attention_layer(6, 1, 14, 0.3),

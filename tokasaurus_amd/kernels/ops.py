@@ -402,6 +402,15 @@ def paged_attention_generic(
     return out
 
 
+def paged_attention_generic_fits(nq: int, nkv: int, head_dim: int, value_dim: int | None = None) -> bool:
+    """Whether the plain 32-bit attention kernel takes this many query heads a kv head at these sizes."""
+    try:
+        call("tk_paged_attention_generic_fits", nq, nkv, head_dim, head_dim if value_dim is None else value_dim)
+    except KernelError:
+        return False
+    return True
+
+
 def attention_mfma_supports(dtype: torch.dtype, head_dim: int, page_size: int) -> bool:
     """Whether the matrix-core attention kernel takes this storage type, head size and page size."""
     return (dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= 128

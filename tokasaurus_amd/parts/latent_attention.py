@@ -50,6 +50,7 @@ class LatentAttention(Mixer):
         ([heads * value_dim, kv_rank]), o ([hidden, heads * value_dim]).  ``key_chunk``: in steps of
         few tokens a request's keys are cut at multiples of this many among workgroups (0: never)."""
         self.key_chunk = int(key_chunk)
+        self.heads_a_call = num_heads  # query heads one call of the plain attention kernel takes (set when the cache is checked)
         self.hidden_size, self.num_heads = hidden_size, num_heads
         self.key_dim, self.value_dim, self.q_rank, self.kv_rank = int(key_dim), int(value_dim), int(q_rank), int(kv_rank)
         self.scale, self.norm_eps = float(scale), float(norm_eps)
@@ -77,8 +78,16 @@ class LatentAttention(Mixer):
         if ops.attention_tile_f32_fits(self.num_heads, 1, self.kv_rank, self.kv_rank, page_size):
             ops.key_pages_shape(1, 1, page_size, self.kv_rank, padded=True)
             ops.value_pages_shape(1, 1, page_size, self.kv_rank)
-        else:  # the plain kernel's bounds (heads times the latent's size)
-            ops.check_attention_shape(dtype, self.num_heads, 1, self.kv_rank, page_size, value_dim=self.kv_rank, generic_only=True)
+        else:
+            # the plain kernel bounds the heads that share a kv head (their number times the latent's size):
+            # more heads than it takes at once go in several calls
+            ops.key_pages_shape(1, 1, page_size, self.kv_rank, padded=True)
+            ops.value_pages_shape(1, 1, page_size, self.kv_rank)
+            m = self.num_heads
+            while m > 1 and not ops.paged_attention_generic_fits(m, 1, self.kv_rank, self.kv_rank):
+                m = (m + 1) // 2
+            ops.check_attention_shape(dtype, m, 1, self.kv_rank, page_size, value_dim=self.kv_rank, generic_only=True)
+            self.heads_a_call = m
 
     def load(self, tensors: dict[str, torch.Tensor], placer: Placer) -> None:
         for lin in (self.down, self.up_q, self.out, self.expand):
@@ -133,8 +142,16 @@ class LatentAttention(Mixer):
                                        key_chunk=self.key_chunk, longest=ctx.extras.get("kv_bound", ctx.max_kv_len),
                                        first_row=first_row)
         else:
-            o = ops.paged_attention_generic(ql, cache.keys, cache.values, cache.block_table, ctx.token_req[first_row:],
-                                            ctx.positions[first_row:], H, 1, r, cache.page_size, scale=self.scale, value_dim=r)
+            o = torch.empty((ql.shape[0], H * r), dtype=ql.dtype, device=ql.device)
+            for h0 in range(0, H, self.heads_a_call):
+                n = min(self.heads_a_call, H - h0)
+                part = ops.paged_attention_generic(ql[:, h0 * r :], cache.keys, cache.values, cache.block_table,
+                                                   ctx.token_req[first_row:], ctx.positions[first_row:], n, 1, r, cache.page_size,
+                                                   scale=self.scale, value_dim=r)
+                if n == H:
+                    o = part
+                else:
+                    o[:, h0 * r : (h0 + n) * r] = part
         return ops.head_linear(o, self.from_latent)  # [rows, heads * value_dim]
 
     def _over_expanded(self, q: torch.Tensor, ctx: StepContext, cache: CacheView, portions: int) -> torch.Tensor:
