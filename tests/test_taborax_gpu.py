@@ -138,13 +138,13 @@ def test_head_linear_and_stream_kernels():
 SINGLE_LAYERS = {
     "latent": latent_layer(4, 16, 24, 20, 32, 0.25),
     "latent_one_head_odd_sizes": latent_layer(1, 12, 7, 9, 21, 0.3),
-    "latent_sizes_of_a_large_model": latent_layer(4, 64, 64, 72, 128, 0.12, dense(96)),
+    "latent_sizes_of_a_large_model": latent_layer(8, 64, 96, 72, 192, 0.12, dense(96)),
     "latent_beyond_the_matrix_core_kernel": latent_layer(2, 16, 16, 24, 272, 0.1),
     "latent_more_heads_than_the_plain_kernel_takes_at_once": latent_layer(9, 8, 16, 16, 264, 0.1),
     "attention_halves_of_a_part": attention_layer(4, 2, 32, 0.18, rot={"base": 100.0, "dims": 12}),
     "attention_whole_head_no_grouping": attention_layer(3, 3, 8, 0.4, rot={"base": 9.0, "dims": 8}),
     "attention_no_rotation_odd_head": attention_layer(6, 1, 14, 0.3),
-    "attention_sizes_of_a_large_model": attention_layer(8, 2, 128, 0.09, rot={"base": 10000.0, "dims": 32}),
+    "attention_sizes_of_a_large_model": attention_layer(8, 2, 128, 0.09, rot={"base": 500000.0, "dims": 64}),
     "dense": attention_layer(1, 1, 8, 1.0, mlp=dense(72)),
     "experts_groups_identity_shared": attention_layer(1, 1, 8, 1.0, mlp=moe(24, 13, 4, identity=3, groups=(4, 3), shared=16)),
     "experts_one_choice": latent_layer(1, 8, 8, 8, 8, 0.5, moe(40, 3, 1)),
