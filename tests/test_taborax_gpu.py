@@ -375,3 +375,54 @@ def test_command_line_and_trace_replay(taborax_folders, tmp_path):
     for step, rows in want.items():
         got = torch.from_numpy(np.fromfile(out / f"{step}.f32", dtype="<f4").reshape(len(rows), vocab).copy())
         compare_rows({key: got[i] for i, key in enumerate(rows)}, plain, TOL["float32"])
+
+
+def random_config(seed: int) -> dict:
+    """A Taborax configuration drawn from lists of sizes that hold the kernels' comfortable values and awkward ones."""
+    import random
+
+    rng = random.Random(seed)
+    width = rng.choice([48, 64, 72, 96, 136])
+    layers = []
+    for _ in range(rng.randint(2, 5)):
+        kind = rng.choice(["dense", "moe", "moe", None])
+        mlp = None
+        if kind == "dense":
+            mlp = dense(rng.choice([40, 64, 100, 160]))
+        elif kind == "moe":
+            experts, identity = rng.randint(2, 12), rng.choice([0, 0, 1, 3])
+            n_all = experts + identity
+            count = rng.choice([g for g in (1, 2, 3, 4, 5) if n_all % g == 0])
+            keep = rng.randint(1, count)
+            top = rng.randint(1, min(4, n_all // count * keep))
+            mlp = moe(rng.choice([8, 20, 32, 48]), experts, top, identity=identity if identity else None,
+                      groups=(count, keep) if rng.random() < 0.8 or count > 1 else None, shared=rng.choice([None, 16, 40]))
+        if rng.random() < 0.5:
+            layers.append(latent_layer(rng.choice([1, 2, 3, 4, 6, 8]), rng.choice([8, 16, 24, 32, 40, 64]), rng.choice([8, 16, 32, 48, 64]),
+                                       rng.choice([8, 12, 24, 40]), rng.choice([8, 16, 24, 48, 64, 80, 128]), rng.uniform(0.05, 0.4), mlp))
+        else:
+            kv, dim = rng.choice([1, 2, 4]), rng.choice([8, 16, 32, 64, 128])
+            rot = None if rng.random() < 0.25 else {"base": rng.choice([10.0, 1000.0, 1e6]), "dims": 2 * rng.randint(1, dim // 2)}
+            layers.append(attention_layer(kv * rng.choice([1, 2, 3, 4]), kv, dim, rng.uniform(0.05, 0.4), rot=rot, mlp=mlp))
+    cfg = {"architecture": "Taborax", "vocab": rng.randint(50, 300), "width": width, "norm": {"eps": rng.choice([1e-6, 1e-5, 1e-3])},
+           "layers": layers}
+    if rng.random() < 0.7:
+        start = rng.randint(0, len(layers) - 1)
+        cfg["loop"] = {"start": start, "stop": rng.randint(start + 1, len(layers)), "times": rng.randint(1, 3)}
+    return cfg
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_configurations(tmp_path, seed):
+    """Drawn configurations in 32-bit: a prompt whole, its tail token by token, in portions, and beside another request."""
+    config = random_config(seed)
+    folder = make_folder(tmp_path / "m", config, seed=seed)
+    reqs = {"a": random_tokens(75, config["vocab"], seed), "b": random_tokens(22, config["vocab"], seed + 100)}
+    plain = plain_rows(folder, reqs)
+    runner = runner_for(folder, "float32", tokens=192)
+    tol = TOL["float32"]
+    compare_rows(run_steps(runner, whole("a", reqs["a"])), plain, tol)
+    compare_rows(run_steps(runner, tail_one_by_one("a", reqs["a"], tail=20)), plain, tol)
+    compare_rows(run_steps(runner, portions("a", reqs["a"], [2, 17, 1, 33, 3])), plain, tol)
+    compare_rows(run_steps(runner, mixed_trace(reqs, seed, max_live=2)), plain, tol)
+    assert runner.manager.requests == {}
